@@ -170,7 +170,8 @@ class CacheManager:
                 continue
             first_needed = max(0, next_position - w + 1)      # oldest position still read
             table = rc.tables[g.index]
-            for pi in range(min(first_needed // self.page_size, len(table))):
+            kept = -(-g.need.keep_first // self.page_size)    # pages of the first tokens, read for ever
+            for pi in range(kept, min(first_needed // self.page_size, len(table))):
                 if table[pi] >= 0:
                     g.pool.free([table[pi]])
                     table[pi] = -1

@@ -110,3 +110,46 @@ def zimorax_preset(name: str, **overrides):
     fields: Dict = dict(vocab=50272, width=hidden, layers=layers, loop=loop, norm_eps=1e-5, max_positions=4096)
     fields.update(overrides)
     return ZimoraxHyperParam(**fields).validate()
+
+
+# ---- named sizes of the Gisedra family, for runs with random weights: the layer sizes of the OPT model of
+# the same name (width, heads).  Of every four layers the third is a parallel pair (window attention with a
+# quarter of the heads as key heads, a window of 1,024 that keeps the first 16 tokens, rotary positions on
+# half of each head; beside it a retention of an eighth of the heads), the others latent attention (rank
+# 128, a rotated part of 32, a window of 1,024); every layer has 16 experts of a quarter of the OPT
+# feed-forward's width, 2 a token, and a token input of 16; the first two layers run twice.
+def gisedra_preset(name: str, **overrides):
+    from .gisedra_param import GisedraHyperParam
+    key = name.lower().replace("-", "_")
+    size = key.split("_", 1)[1] if "_" in key else ""
+    if "opt_" + size not in _SIZES:
+        raise KeyError(f"invalid model name {name!r}; valid names: " +
+                       " ".join("gisedra_" + k.split("_", 1)[1] for k in _SIZES))
+    n_layers, hidden, heads, ffn = _SIZES["opt_" + size]
+    n_layers = int(overrides.pop("num_layers", n_layers))
+    only = overrides.pop("only", None)            # one mixer type for every layer (measurements)
+    window = int(overrides.pop("window", 1024))
+    loop_times = int(overrides.pop("loop_times", 2))
+    hd = hidden // heads
+    layers = []
+    for i in range(n_layers):
+        kind = only or ("latent_attention", "latent_attention", "parallel", "latent_attention")[i % 4]
+        if kind == "latent_attention":
+            mixer = {"heads": heads, "dim": hd, "rot_dim": 32, "vdim": hd, "kv_rank": 128,
+                     "scale": float(hd + 32) ** -0.5, "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 32}}
+        else:
+            rh = max(1, heads // 8)
+            mixer = {"left_scale": 1.0, "right_scale": 1.0,
+                     "left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": hd, "vdim": hd,
+                              "scale": float(hd) ** -0.5, "conv": 4, "mask": {"size": window, "keep_first": 16},
+                              "rot": {"dims": hd // 2, "base": 10000.0,
+                                      "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}},
+                     "right": {"heads": rh, "dim": hd, "vdim": 2 * hd,
+                               "decay": [1.0 - 2.0 ** (-5 - (j % 4)) for j in range(rh)]}}
+        mlp = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ffn // 4}}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    loop = {"start": 0, "stop": min(2, n_layers), "times": loop_times} if loop_times > 0 else None
+    fields: Dict = dict(vocab=50272, width=hidden, layers=layers, loop=loop, token_side_dim=16, norm_eps=1e-5,
+                        max_positions=4096)
+    fields.update(overrides)
+    return GisedraHyperParam(**fields).validate()

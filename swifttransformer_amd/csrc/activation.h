@@ -6,14 +6,15 @@
 // The reference has the same three (src/csrc/kernel/activations.cuh:8-24): ReLU, SiLU as
 // x / (1 + exp(-x)), and GELU in its tanh form 0.5 x (1 + tanh(0.79788456 (x + 0.044715 x^3))).
 // Here they are always evaluated in float, with the accurate exp and tanh.  A fourth, GELU in its
-// exact form 0.5 x (1 + erf(x / sqrt 2)), and a fifth, the square of ReLU, have no counterpart there.
+// exact form 0.5 x (1 + erf(x / sqrt 2)), a fifth, the square of ReLU, and a sixth, the logistic
+// function 1 / (1 + exp(-x)) (a gate), have no counterpart there.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <math.h>
 
 namespace st {
 
-enum Activation : int { kActNone = 0, kActRelu = 1, kActSilu = 2, kActGeluTanh = 3, kActGeluErf = 4, kActReluSquared = 5, kNumActivations };
+enum Activation : int { kActNone = 0, kActRelu = 1, kActSilu = 2, kActGeluTanh = 3, kActGeluErf = 4, kActReluSquared = 5, kActSigmoid = 6, kNumActivations };
 
 inline bool activation_known(int kind) { return kind >= 0 && kind < kNumActivations; }
 // the vendor library's epilogues are asked for these only; the others run in this library's kernels
@@ -26,6 +27,7 @@ __host__ __device__ inline float apply_activation(int kind, float v) {
         case kActGeluTanh: return 0.5f * v * (1.f + tanhf(0.79788456f * (v + 0.044715f * v * v * v)));
         case kActGeluErf: return 0.5f * v * (1.f + erff(0.70710678f * v));
         case kActReluSquared: { const float r = fmaxf(v, 0.f); return r * r; }
+        case kActSigmoid: return 1.f / (1.f + expf(-v));
         default: return v;
     }
 }

@@ -113,11 +113,12 @@ int st_token_conv_state(float* state, int64_t slot_stride, const void* x, int64_
                         int channels, int taps, hipStream_t stream);
 
 // ---- rotary positions, one-pool page write, two float rows side by side in the storage type (csrc/rotary.hip)
-// In place on the rows' queries and keys: the first rot_dims coordinates of every head, coordinate i
-// paired with i + rot_dims / 2, turned by positions[t] * freq[i]; cosine and sine times `mult`.
+// In place on the rows' queries and keys: the rot_dims coordinates of every head from `offset` on,
+// coordinate i paired with i + rot_dims / 2 (interleaved != 0: 2i with 2i + 1), turned by
+// positions[t] * freq[i]; cosine and sine times `mult`.
 int st_rotary(void* q, int64_t q_stride, int q_heads, void* k, int64_t k_stride, int k_heads, int head_dim,
-              int rot_dims, const float* freq, float mult, const int* positions, int num_tokens, int dtype,
-              hipStream_t stream);
+              int rot_dims, int offset, int interleaved, const float* freq, float mult, const int* positions,
+              int num_tokens, int dtype, hipStream_t stream);
 // src[t, head, :] -> the token's entry of a pool [pages, heads, page_size, head_dim]; norm != 0: divided
 // by its root mean square over head_dim (eps inside the root) on the way.
 int st_paged_write(void* cache, int64_t page_stride, const void* src, int64_t src_stride, const int* token_item,
@@ -132,7 +133,8 @@ int st_sink_attention(void* out, float* part_o, float* part_ml, const void* q, i
                       const void* k_cache, int64_t k_page_stride, const void* v_cache, int64_t v_page_stride,
                       const float* mix, const int* token_item, const int* positions, const int* block_table,
                       int max_pages, int page_size, int num_tokens, int heads, int kv_heads, int key_dim,
-                      int value_dim, float scale, int window, int sink, int splits, int dtype, hipStream_t stream);
+                      int value_dim, float scale, int window, int keep_first, int sink, int splits, int dtype,
+                      hipStream_t stream);
 
 // ---- recurrences with one decay a head and token (csrc/state_scan.hip)
 // mode 0: out_a = softplus(raw + bias), out_b = exp(-exp(a_log) * out_a), raw [T, heads];
@@ -143,10 +145,11 @@ int st_recurrence_gates(float* out_a, float* out_b, const float* raw, int64_t ra
 int st_unit_norm(float* x, int64_t stride, int num_tokens, int heads, int dim, float eps, float scale,
                  hipStream_t stream);
 // mode 0: S <- b S + (a k) v^T, o = S^T q + skip v;  mode 1: S <- b S, u = a (v - S^T k), S <- S + k u^T,
-// o = S^T q.  a, b float [T, heads]; q, k float rows of qk_heads heads; state [slots](slot_stride)
-// [heads, key_dim, value_dim] float.
+// o = S^T q.  a, b float [T, heads] with rows gate_stride floats apart (0: one row of constants serves
+// every token); q, k float rows of qk_heads heads; state [slots](slot_stride) [heads, key_dim, value_dim] float.
 int st_state_scan(float* out, const float* q, int64_t q_stride, const float* k, int64_t k_stride, const float* v,
-                  int64_t v_stride, const float* gate_a, const float* gate_b, const float* skip, float* state,
+                  int64_t v_stride, const float* gate_a, const float* gate_b, int64_t gate_stride, const float* skip,
+                  float* state,
                   int64_t slot_stride, const int* item_len, const int* item_tok_off, const int* item_slot,
                   int num_items, int max_item_rows, int heads, int qk_heads, int key_dim, int value_dim, int mode,
                   hipStream_t stream);
@@ -180,16 +183,20 @@ int st_gated_head_norm(void* out, const float* o, int parts, int64_t part_stride
 // ---- latent cache (csrc/latent.hip)
 // Row t of x (float, stride x_stride, `rank` values) is normalised, c = x * rsqrt(mean x^2 + eps) *
 // gain, and stored as the token's entry of a one-head page pool whose entries are `entry` >= rank
-// wide (the rest is cleared): [pages, 1, page_size, entry] of `dtype`.
+// wide (the rest is cleared): [pages, 1, page_size, entry] of `dtype`.  tail > 0: the row's next `tail`
+// values follow the latent in the entry as they are, or, with `freq` [tail / 2], turned by the token's
+// position (pairs 2i, 2i + 1; angle position * freq[i]): a key part that every head shares.
 int st_latent_write(void* cache, int64_t page_stride, const float* x, int64_t x_stride, const float* gain,
                     const int* token_item, const int* positions, const int* block_table, int max_pages,
-                    int page_size, int num_tokens, int rank, int entry, float eps, int dtype, hipStream_t stream);
+                    int page_size, int num_tokens, int rank, int entry, float eps, int tail, const float* freq,
+                    int dtype, hipStream_t stream);
 
 // ---- routed experts (csrc/moe.hip)
 // ids[t, j], weights[t, j] (j < top): the experts with the largest logits of row t, largest first,
-// the lower index on ties, and sigmoid of their logits.  Rows whose item is -1 get ids of -1.
+// the lower index on ties, and their weights: mode 0 the sigmoid of each logit, mode 1 the softmax over
+// the chosen logits alone.  Rows whose item is -1 get ids of -1.
 int st_moe_route(int* ids, float* weights, const float* logits, const int* token_item, int num_tokens,
-                 int experts, int top, hipStream_t stream);
+                 int experts, int top, int mode, hipStream_t stream);
 // Sorts the num_pairs = tokens * top (token, choice) pairs by expert into tiles of `tile` (16, 64 or 128)
 // places that hold one expert's pairs each: sorted[capacity] (pair index, or -1),
 // place_of_pair[num_pairs] (or -1), tile_expert[capacity / tile] (or -1).
@@ -198,18 +205,32 @@ int st_moe_align(int* sorted, int* place_of_pair, int* tile_expert, const int* i
                  int experts, int capacity, int tile, hipStream_t stream);
 // y[place, f] = g * sigmoid(1.702 g) * (u + 1) with g = min(s * (x_t . Wg[e, f]), limit) and
 // u = clamp(s * (x_t . Wu[e, f]), -limit, limit), for the pair (t, j) at `place`, e its expert and s
-// its weight.  x: [T, width]; w_gate, w_up: [experts, inner, width]; y: [capacity, inner].
+// its weight (style 0); style 1: y[place, f] = silu(x_t . Wg[e, f]) * (x_t . Wu[e, f]), no weight and no
+// limit (the weight then multiplies the expert's result, in st_moe_combine).
+// x: [T, width]; w_gate, w_up: [experts, inner, width]; y: [capacity, inner].
 int st_moe_up(void* y, const void* x, const void* w_gate, const void* w_up, const int* sorted,
               const int* tile_expert, const float* weights, int capacity, int tile, int top, int width, int inner,
-              float limit, int dtype, hipStream_t stream);
+              float limit, int style, int dtype, hipStream_t stream);
 // pair_out[place, n] = y[place] . Wd[e, n] (top > 1), or, with top == 1, directly
 // out[t, n] = residual[t, n] + out_scale * y[place] . Wd[e, n].  w_down: [experts, width, inner].
 int st_moe_down(float* out, const float* residual, float* pair_out, const void* y, const void* w_down,
                 const int* sorted, const int* tile_expert, int capacity, int tile, int top, int width, int inner,
                 float out_scale, int dtype, hipStream_t stream);
-// out[t, n] = residual[t, n] + out_scale * sum_j pair_out[place_of_pair[t * top + j], n]
+// out[t, n] = residual[t, n] + out_scale * sum_j weights[t * top + j] * pair_out[place_of_pair[t * top + j], n]
+// (weights null: ones; residual null: zeros)
 int st_moe_combine(float* out, const float* residual, const float* pair_out, const int* place_of_pair,
-                   int num_tokens, int top, int width, float out_scale, hipStream_t stream);
+                   const float* weights, int num_tokens, int top, int width, float out_scale, hipStream_t stream);
+
+// ---- float operations on the residual stream (csrc/stream_ops.hip)
+// y = tanh(alpha[0] * x[row]) * w + b (b may be null) of every row, or of the rows picked by `rows`
+// (negative: skipped); base != null: y += base[row of the result]; out32 (float) and / or out_t (`dtype`).
+int st_dynamic_tanh(void* out_t, float* out32, const float* x, const int* rows, const float* w, const float* b,
+                    const float* alpha, const float* base, int num_rows, int width, int dtype, hipStream_t stream);
+// x[t] += y[t] * rsqrt(mean(y[t]^2) + eps) * w
+int st_unit_add(float* x, const float* y, const float* w, int num_rows, int width, float eps, hipStream_t stream);
+// out[t] = x[t] (+ first[t]) + vec
+int st_row_add(float* out, const float* x, const float* first, const float* vec, int num_rows, int width,
+               hipStream_t stream);
 
 // Measurement kernels (csrc/probe.hip): a plain streaming read, and a kernel without work.
 int st_probe_read(const void* src, int64_t bytes, void* sink, int workgroups, int pattern, hipStream_t stream);

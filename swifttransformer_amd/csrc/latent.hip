@@ -13,7 +13,7 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
     T* __restrict__ cache, int64_t page_stride, const float* __restrict__ x, int64_t x_stride,
     const float* __restrict__ gain, const int* __restrict__ token_item, const int* __restrict__ positions,
     const int* __restrict__ block_table, int max_pages, int page_size, int num_tokens, int rank, int entry,
-    float eps) {
+    float eps, int tail, const float* __restrict__ freq) {
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= num_tokens) return;
@@ -27,8 +27,23 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
     ss = wave_sum(ss);
     const float r = 1.f / sqrtf(ss / (float)rank + eps);
     T* dst = cache + (int64_t)page * page_stride + (int64_t)(pos % page_size) * entry;
-    for (int j = lane; j < entry; j += 64)
-        Elem<T>::store(dst + j, j < rank ? xp[j] * r * gain[j] : 0.f);
+    for (int j = lane; j < entry; j += 64) {
+        float v = 0.f;
+        if (j < rank) {
+            v = xp[j] * r * gain[j];
+        } else if (j < rank + tail) {
+            v = xp[j];
+            if (freq) {                               // pairs (2i, 2i + 1) of the tail turn with the position
+                const int i = (j - rank) >> 1;
+                const float a = (float)pos * freq[i];
+                const float c = cosf(a), s = sinf(a);
+                const int ju = rank + 2 * i;
+                const float u = xp[ju], w = xp[ju + 1];
+                v = ((j - rank) & 1) ? w * c + u * s : u * c - w * s;
+            }
+        }
+        Elem<T>::store(dst + j, v);
+    }
 }
 
 }  // namespace st
@@ -37,19 +52,21 @@ using namespace st;
 
 extern "C" int st_latent_write(void* cache, int64_t page_stride, const float* x, int64_t x_stride, const float* gain,
                                const int* token_item, const int* positions, const int* block_table, int max_pages,
-                               int page_size, int num_tokens, int rank, int entry, float eps, int dtype,
-                               hipStream_t stream) {
-    ST_CHECK(num_tokens >= 0 && rank > 0 && entry >= rank && page_size > 0 && max_pages > 0, "latent_write: bad sizes");
+                               int page_size, int num_tokens, int rank, int entry, float eps, int tail,
+                               const float* freq, int dtype, hipStream_t stream) {
+    ST_CHECK(num_tokens >= 0 && rank > 0 && tail >= 0 && entry >= rank + tail && page_size > 0 && max_pages > 0,
+             "latent_write: bad sizes");
+    ST_CHECK(!freq || tail % 2 == 0, "latent_write: a turned tail has an even size");
     ST_CHECK(cache && x && gain && token_item && positions && block_table, "latent_write: null operand");
     ST_CHECK(eps > 0.f, "latent_write: eps must be positive");
     if (num_tokens == 0) return 0;
     const unsigned grid = (unsigned)((num_tokens + 3) / 4);
     if (dtype == kF32)
         latent_write_kernel<float><<<grid, 256, 0, stream>>>((float*)cache, page_stride, x, x_stride, gain, token_item,
-            positions, block_table, max_pages, page_size, num_tokens, rank, entry, eps);
+            positions, block_table, max_pages, page_size, num_tokens, rank, entry, eps, tail, freq);
     else if (dtype == kBF16)
         latent_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)cache, page_stride, x, x_stride, gain, token_item,
-            positions, block_table, max_pages, page_size, num_tokens, rank, entry, eps);
+            positions, block_table, max_pages, page_size, num_tokens, rank, entry, eps, tail, freq);
     else ST_CHECK(false, "latent_write: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("latent_write");
     return 0;

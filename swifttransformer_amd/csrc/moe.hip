@@ -26,7 +26,7 @@ constexpr int kMaxTop = 16;
 
 __global__ __launch_bounds__(256) void moe_route_kernel(
     int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ logits,
-    const int* __restrict__ token_item, int num_tokens, int experts, int top) {
+    const int* __restrict__ token_item, int num_tokens, int experts, int top, int mode) {
     const int t = blockIdx.x * 256 + threadIdx.x;
     if (t >= num_tokens) return;
     if (token_item && token_item[t] < 0) {
@@ -46,7 +46,15 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
         }
         chosen[j] = best;
         ids[(int64_t)t * top + j] = best;
-        weights[(int64_t)t * top + j] = 1.f / (1.f + expf(-bv));
+        weights[(int64_t)t * top + j] = mode == 0 ? 1.f / (1.f + expf(-bv)) : bv;
+    }
+    if (mode == 1) {
+        // softmax over the chosen logits alone; the first chosen is the largest
+        float* w = weights + (int64_t)t * top;
+        const float m = w[0];
+        float sum = 0.f;
+        for (int j = 0; j < top; ++j) { w[j] = expf(w[j] - m); sum += w[j]; }
+        for (int j = 0; j < top; ++j) w[j] /= sum;
     }
 }
 
@@ -143,7 +151,7 @@ template <typename T, int RT>
 __global__ __launch_bounds__(256) void moe_up_kernel(
     T* __restrict__ y, const T* __restrict__ x, const T* __restrict__ w_gate, const T* __restrict__ w_up,
     const int* __restrict__ sorted, const int* __restrict__ tile_expert, const float* __restrict__ weights,
-    int top, int width, int inner, float limit, int vec) {
+    int top, int width, int inner, float limit, int style, int vec) {
     const int tile = blockIdx.x;
     const int e = tile_expert[tile];
     if (e < 0) return;
@@ -187,7 +195,10 @@ __global__ __launch_bounds__(256) void moe_up_kernel(
             const int place = base + b * kRows + 4 * g + r;
             const int p = sorted[place];
             float out = 0.f;
-            if (p >= 0) {
+            if (p >= 0 && style == 1) {
+                const float gv = cg[b][r];
+                out = gv / (1.f + expf(-gv)) * cu[b][r];
+            } else if (p >= 0) {
                 const float s = weights[p];
                 const float gv = fminf(s * cg[b][r], limit);
                 const float uv = fminf(fmaxf(s * cu[b][r], -limit), limit);
@@ -261,7 +272,7 @@ __global__ __launch_bounds__(256) void moe_tiled_kernel(
     bf16_t* __restrict__ y_out, float* __restrict__ out, const float* __restrict__ residual,
     float* __restrict__ pair_out, const bf16_t* __restrict__ a_rows, const bf16_t* __restrict__ w0,
     const bf16_t* __restrict__ w1, const int* __restrict__ sorted, const int* __restrict__ tile_expert,
-    const float* __restrict__ weights, int top, int N, int K, float limit, float out_scale) {
+    const float* __restrict__ weights, int top, int N, int K, float limit, float out_scale, int style) {
     __shared__ uint4 sw[128 * 8];      // weight rows: [row][chunk of 8 in depth]
     __shared__ uint4 sx[128 * 8];      // places
     const int tile = blockIdx.x;
@@ -339,7 +350,7 @@ __global__ __launch_bounds__(256) void moe_tiled_kernel(
         const int place = base + wm * 64 + j * 32 + l32;
         const int p = sorted[place];
         if (UP) {
-            const float s = p >= 0 ? weights[p] : 0.f;
+            const float s = p >= 0 && style == 0 ? weights[p] : 0.f;
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
                 const int f = n0 + wn * 32 + 8 * q4 + 4 * lh;
@@ -347,6 +358,11 @@ __global__ __launch_bounds__(256) void moe_tiled_kernel(
                 float r[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
+                    if (style == 1) {
+                        const float gv = acc[0][j][4 * q4 + u];
+                        r[u] = p >= 0 ? gv / (1.f + expf(-gv)) * acc[1][j][4 * q4 + u] : 0.f;
+                        continue;
+                    }
                     const float gv = fminf(s * acc[0][j][4 * q4 + u], limit);
                     const float uv = fminf(fmaxf(s * acc[1][j][4 * q4 + u], -limit), limit);
                     r[u] = p >= 0 ? gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f) : 0.f;
@@ -380,17 +396,22 @@ __global__ __launch_bounds__(256) void moe_tiled_kernel(
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     float* __restrict__ out, const float* __restrict__ residual, const float* __restrict__ pair_out,
-    const int* __restrict__ place_of_pair, int top, int width, float out_scale) {
+    const int* __restrict__ place_of_pair, const float* __restrict__ weights, int top, int width, float out_scale) {
     const int t = blockIdx.x;
     for (int n = threadIdx.x; n < width; n += 256) {
         float sum = 0.f;
         bool any = false;
         for (int j = 0; j < top; ++j) {
             const int place = place_of_pair[(int64_t)t * top + j];
-            if (place >= 0) { sum += pair_out[(int64_t)place * width + n]; any = true; }
+            if (place >= 0) {
+                const float v = pair_out[(int64_t)place * width + n];
+                sum = weights ? fmaf(weights[(int64_t)t * top + j], v, sum) : sum + v;
+                any = true;
+            }
         }
         const int64_t at = (int64_t)t * width + n;
-        if (any) out[at] = fmaf(out_scale, sum, residual[at]);
+        if (!residual) out[at] = any ? out_scale * sum : 0.f;
+        else if (any) out[at] = fmaf(out_scale, sum, residual[at]);
         else if (out != residual) out[at] = residual[at];
     }
 }
@@ -400,14 +421,15 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
 using namespace st;
 
 extern "C" int st_moe_route(int* ids, float* weights, const float* logits, const int* token_item, int num_tokens,
-                            int experts, int top, hipStream_t stream) {
+                            int experts, int top, int mode, hipStream_t stream) {
+    ST_CHECK(mode == 0 || mode == 1, "moe_route: mode 0 (sigmoid of each) or 1 (softmax over the chosen)");
     ST_CHECK(num_tokens >= 0 && experts > 0, "moe_route: bad sizes");
     ST_CHECK(top >= 1 && top <= kMaxTop && top <= experts, "moe_route: 1 to %d experts a token (of %d), not %d",
              kMaxTop, experts, top);
     ST_CHECK(ids && weights && logits, "moe_route: null operand");
     if (num_tokens == 0) return 0;
     moe_route_kernel<<<(num_tokens + 255) / 256, 256, 0, stream>>>(ids, weights, logits, token_item, num_tokens,
-                                                                  experts, top);
+                                                                  experts, top, mode);
     ST_LAUNCH_CHECK("moe_route");
     return 0;
 }
@@ -434,8 +456,9 @@ static bool rows_vectorised(const void* a, const void* b, const void* c, int dep
 
 extern "C" int st_moe_up(void* y, const void* x, const void* w_gate, const void* w_up, const int* sorted,
                          const int* tile_expert, const float* weights, int capacity, int tile, int top, int width,
-                         int inner, float limit, int dtype, hipStream_t stream) {
+                         int inner, float limit, int style, int dtype, hipStream_t stream) {
     const int kTile = tile;
+    ST_CHECK(style == 0 || style == 1, "moe_up: style 0 (weighted, clamped inputs) or 1 (plain gated unit)");
     ST_CHECK(tile == 16 || tile == 64 || tile == 128, "moe_up: tiles of 16, 64 or 128 places, not %d", tile);
     ST_CHECK(capacity > 0 && capacity % kTile == 0 && top >= 1 && width > 0 && inner > 0, "moe_up: bad sizes");
     ST_CHECK(y && x && w_gate && w_up && sorted && tile_expert && weights, "moe_up: null operand");
@@ -445,13 +468,13 @@ extern "C" int st_moe_up(void* y, const void* x, const void* w_gate, const void*
     if (dtype == kBF16 && tile == 128 && vec) {
         const dim3 g2(capacity / 128, (inner + 63) / 64);
         moe_tiled_kernel<true><<<g2, 256, 0, stream>>>((bf16_t*)y, nullptr, nullptr, nullptr, (const bf16_t*)x,
-            (const bf16_t*)w_gate, (const bf16_t*)w_up, sorted, tile_expert, weights, top, inner, width, limit, 1.f);
+            (const bf16_t*)w_gate, (const bf16_t*)w_up, sorted, tile_expert, weights, top, inner, width, limit, 1.f, style);
         ST_LAUNCH_CHECK("moe_up (tiled)");
         return 0;
     }
 #define ST_UP(T, RT)                                                                                         \
     moe_up_kernel<T, RT><<<grid, 256, 0, stream>>>((T*)y, (const T*)x, (const T*)w_gate, (const T*)w_up, sorted, \
-                                                   tile_expert, weights, top, width, inner, limit, vec)
+                                                   tile_expert, weights, top, width, inner, limit, style, vec)
     if (dtype == kF32) { if (tile == 16) ST_UP(float, 1); else if (tile == 64) ST_UP(float, 4); else ST_UP(float, 8); }
     else if (dtype == kBF16) { if (tile == 16) ST_UP(bf16_t, 1); else if (tile == 64) ST_UP(bf16_t, 4); else ST_UP(bf16_t, 8); }
     else ST_CHECK(false, "moe_up: unknown dtype %d", dtype);
@@ -475,7 +498,7 @@ extern "C" int st_moe_down(float* out, const float* residual, float* pair_out, c
     if (dtype == kBF16 && tile == 128 && vec) {
         const dim3 g2(capacity / 128, (width + 127) / 128);
         moe_tiled_kernel<false><<<g2, 256, 0, stream>>>(nullptr, out, residual, pair_out, (const bf16_t*)y,
-            (const bf16_t*)w_down, nullptr, sorted, tile_expert, nullptr, top, width, inner, 0.f, out_scale);
+            (const bf16_t*)w_down, nullptr, sorted, tile_expert, nullptr, top, width, inner, 0.f, out_scale, 0);
         ST_LAUNCH_CHECK("moe_down (tiled)");
         return 0;
     }
@@ -491,11 +514,12 @@ extern "C" int st_moe_down(float* out, const float* residual, float* pair_out, c
 }
 
 extern "C" int st_moe_combine(float* out, const float* residual, const float* pair_out, const int* place_of_pair,
-                              int num_tokens, int top, int width, float out_scale, hipStream_t stream) {
+                              const float* weights, int num_tokens, int top, int width, float out_scale,
+                              hipStream_t stream) {
     ST_CHECK(num_tokens >= 0 && top >= 1 && width > 0, "moe_combine: bad sizes");
-    ST_CHECK(out && residual && pair_out && place_of_pair, "moe_combine: null operand");
+    ST_CHECK(out && pair_out && place_of_pair, "moe_combine: null operand");
     if (num_tokens == 0) return 0;
-    moe_combine_kernel<<<num_tokens, 256, 0, stream>>>(out, residual, pair_out, place_of_pair, top, width, out_scale);
+    moe_combine_kernel<<<num_tokens, 256, 0, stream>>>(out, residual, pair_out, place_of_pair, weights, top, width, out_scale);
     ST_LAUNCH_CHECK("moe_combine");
     return 0;
 }

@@ -1,8 +1,8 @@
 // Rotary position encoding on the queries and keys of a step, in place, and the write of one
 // paged pool (keys, or values with an optional per-head unit norm) from a step's rows.
 //
-// Rotation: of every head the first `rot_dims` coordinates are turned, coordinate i paired with
-// i + rot_dims / 2:  (u, v) -> (u c - v s, v c + u s),  c = m cos(p f_i), s = m sin(p f_i), p the
+// Rotation: of every head the `rot_dims` coordinates from `offset` on are turned, coordinate i paired with
+// i + rot_dims / 2 (or, `interleaved`, 2i with 2i + 1):  (u, v) -> (u c - v s, v c + u s),  c = m cos(p f_i), s = m sin(p f_i), p the
 // row's position, f the table of angles a position step (any scaling of the frequencies is in the
 // table), m a factor on both.  Position, angle, cosine and sine are float.
 #include "api.h"
@@ -13,8 +13,8 @@ namespace st {
 template <typename T>
 __global__ __launch_bounds__(256) void rotary_kernel(
     T* __restrict__ q, int64_t q_stride, int q_heads, T* __restrict__ k, int64_t k_stride, int k_heads,
-    int head_dim, int half, const float* __restrict__ freq, float mult, const int* __restrict__ positions,
-    int64_t total) {
+    int head_dim, int half, int offset, int interleaved, const float* __restrict__ freq, float mult,
+    const int* __restrict__ positions, int64_t total) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     const int per_row = (q_heads + k_heads) * half;
@@ -23,13 +23,14 @@ __global__ __launch_bounds__(256) void rotary_kernel(
     const int head = r / half, i = r - head * half;
     const int pos = positions[t];
     if (pos < 0) return;                               // a padding row
-    T* p = head < q_heads ? q + t * q_stride + (int64_t)head * head_dim
-                          : k + t * k_stride + (int64_t)(head - q_heads) * head_dim;
+    T* p = (head < q_heads ? q + t * q_stride + (int64_t)head * head_dim
+                           : k + t * k_stride + (int64_t)(head - q_heads) * head_dim) + offset;
     const float a = (float)pos * freq[i];
     const float c = cosf(a) * mult, s = sinf(a) * mult;
-    const float u = Elem<T>::load(p + i), v = Elem<T>::load(p + i + half);
-    Elem<T>::store(p + i, u * c - v * s);
-    Elem<T>::store(p + i + half, v * c + u * s);
+    const int iu = interleaved ? 2 * i : i, iv = interleaved ? 2 * i + 1 : i + half;
+    const float u = Elem<T>::load(p + iu), v = Elem<T>::load(p + iv);
+    Elem<T>::store(p + iu, u * c - v * s);
+    Elem<T>::store(p + iv, v * c + u * s);
 }
 
 // a wave a (row, head): src[t, head, :] (optionally divided by its root mean square) -> its page entry
@@ -80,11 +81,11 @@ __global__ __launch_bounds__(256) void concat_cast_kernel(T* __restrict__ out, c
 using namespace st;
 
 extern "C" int st_rotary(void* q, int64_t q_stride, int q_heads, void* k, int64_t k_stride, int k_heads,
-                         int head_dim, int rot_dims, const float* freq, float mult, const int* positions,
-                         int num_tokens, int dtype, hipStream_t stream) {
+                         int head_dim, int rot_dims, int offset, int interleaved, const float* freq, float mult,
+                         const int* positions, int num_tokens, int dtype, hipStream_t stream) {
     ST_CHECK(num_tokens >= 0 && q_heads >= 0 && k_heads >= 0 && head_dim > 0, "rotary: bad sizes");
-    ST_CHECK(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= head_dim, "rotary: %d turned coordinates in heads of %d",
-             rot_dims, head_dim);
+    ST_CHECK(rot_dims >= 0 && rot_dims % 2 == 0 && offset >= 0 && offset + rot_dims <= head_dim,
+             "rotary: %d turned coordinates from %d on in heads of %d", rot_dims, offset, head_dim);
     if (num_tokens == 0 || rot_dims == 0 || q_heads + k_heads == 0) return 0;
     ST_CHECK((q || q_heads == 0) && (k || k_heads == 0) && freq && positions, "rotary: null operand");
     const int half = rot_dims / 2;
@@ -92,10 +93,10 @@ extern "C" int st_rotary(void* q, int64_t q_stride, int q_heads, void* k, int64_
     const unsigned grid = (unsigned)((total + 255) / 256);
     if (dtype == kF32)
         rotary_kernel<float><<<grid, 256, 0, stream>>>((float*)q, q_stride, q_heads, (float*)k, k_stride, k_heads,
-                                                       head_dim, half, freq, mult, positions, total);
+                                                       head_dim, half, offset, interleaved, freq, mult, positions, total);
     else if (dtype == kBF16)
         rotary_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)q, q_stride, q_heads, (bf16_t*)k, k_stride, k_heads,
-                                                        head_dim, half, freq, mult, positions, total);
+                                                        head_dim, half, offset, interleaved, freq, mult, positions, total);
     else ST_CHECK(false, "rotary: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("rotary");
     return 0;

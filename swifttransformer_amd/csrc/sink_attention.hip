@@ -4,6 +4,7 @@
 //   r_g(i, j)  = scale * q_g(i) . k_c(g)(j)                  c(g) = g / (heads / kv_heads)
 //   s_h(i, j)  = sum_g M[h, g] r_g(i, j)                     (M null: s = r)
 //   p_h(i, j)  = exp(s_h(i, j)) / (sink + sum_j' exp(s_h(i, j')))      over max(0, i - window + 1) <= j' <= i
+//                and, with keep_first > 0, over j' < keep_first as well (the first tokens stay visible)
 //   o_h(i)     = sum_j p_h(i, j) v_c(h)(j)
 //
 // sink = 1 puts a key of score 0 and no value into every row's sum (its softmax starts from the
@@ -32,7 +33,7 @@ struct SinkAttnArgs {
     const void* v_cache; int64_t v_page_stride;
     const float* mix;          // [heads, heads] or null
     const int* token_item; const int* positions; const int* block_table;
-    int max_pages, page_size, heads, kv_heads, key_dim, value_dim, window, sink, splits;
+    int max_pages, page_size, heads, kv_heads, key_dim, value_dim, window, keep_first, sink, splits;
     float scale;
 };
 
@@ -135,16 +136,19 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
         ov[i] = (oh[i] / per) * a.page_size * dv + (e - oh[i] * dv);
     }
     const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-    // this split's share of the row's key blocks
-    const int blocks = (pos - lo) / kKeyBlock + 1;
+    // the row's key blocks: those of the first tokens that stay visible behind the window (positions
+    // below both keep_first and lo), then those of the window; this split's share of them
+    const int kept = min(a.keep_first, lo);
+    const int kept_blocks = (kept + kKeyBlock - 1) / kKeyBlock;
+    const int blocks = kept_blocks + (pos - lo) / kKeyBlock + 1;
     const int share = (blocks + a.splits - 1) / a.splits;
     const int b0 = split * share, b1 = min(blocks, b0 + share);
     const int* bt = a.block_table + (int64_t)item * a.max_pages;
     const T* kc = (const T*)a.k_cache;
     const T* vc = (const T*)a.v_cache;
     for (int b = b0; b < b1; ++b) {
-        const int j0 = lo + b * kKeyBlock;
-        const int nk = min(kKeyBlock, pos - j0 + 1);
+        const int j0 = b < kept_blocks ? b * kKeyBlock : lo + (b - kept_blocks) * kKeyBlock;
+        const int nk = min(kKeyBlock, (b < kept_blocks ? kept : pos + 1) - j0);
         __syncthreads();                           // the block before is done with the shared lists
         if (tid < kKeyBlock) {
             const int j = j0 + (tid < nk ? tid : 0), pi = j / a.page_size;
@@ -350,11 +354,11 @@ extern "C" int st_sink_attention(void* out, float* part_o, float* part_ml, const
                                  const void* k_cache, int64_t k_page_stride, const void* v_cache,
                                  int64_t v_page_stride, const float* mix, const int* token_item, const int* positions,
                                  const int* block_table, int max_pages, int page_size, int num_tokens, int heads,
-                                 int kv_heads, int key_dim, int value_dim, float scale, int window, int sink,
-                                 int splits, int dtype, hipStream_t stream) {
+                                 int kv_heads, int key_dim, int value_dim, float scale, int window, int keep_first,
+                                 int sink, int splits, int dtype, hipStream_t stream) {
     ST_CHECK(num_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && key_dim > 0 && value_dim > 0,
              "sink_attention: bad sizes");
-    ST_CHECK(page_size > 0 && max_pages > 0 && window >= 0 && splits >= 1 && splits <= 16, "sink_attention: 1 to 16 splits");
+    ST_CHECK(page_size > 0 && max_pages > 0 && window >= 0 && keep_first >= 0 && splits >= 1 && splits <= 16, "sink_attention: 1 to 16 splits");
     ST_CHECK(heads <= 256, "sink_attention: up to 256 heads, not %d", heads);
     ST_CHECK(heads * value_dim <= 32 * 256, "sink_attention: heads x value size up to 8192, not %d", heads * value_dim);
     const int64_t lds_bytes = st_sink_attention_lds(heads, key_dim, mix != nullptr);
@@ -368,7 +372,7 @@ extern "C" int st_sink_attention(void* out, float* part_o, float* part_ml, const
     a.k_cache = k_cache; a.k_page_stride = k_page_stride; a.v_cache = v_cache; a.v_page_stride = v_page_stride;
     a.mix = mix; a.token_item = token_item; a.positions = positions; a.block_table = block_table;
     a.max_pages = max_pages; a.page_size = page_size; a.heads = heads; a.kv_heads = kv_heads;
-    a.key_dim = key_dim; a.value_dim = value_dim; a.window = window; a.sink = sink; a.splits = splits;
+    a.key_dim = key_dim; a.value_dim = value_dim; a.window = window; a.keep_first = keep_first; a.sink = sink; a.splits = splits;
     a.scale = scale;
     if (dtype == kF32) return launch_sink_attention<float>(a, num_tokens, (size_t)lds_bytes, stream);
     if (dtype == kBF16) return launch_sink_attention<bf16_t>(a, num_tokens, (size_t)lds_bytes, stream);

@@ -6,7 +6,7 @@
 //                                    S <- S + k_t u^T;                      o_t = S^T q_t
 //
 // a_t (the decay) and b_t (the step size, or the write strength) are float [T, heads] made by
-// `recurrence_gates`; q, k, v are float rows; the state is float, lives in the request's slot and is
+// `recurrence_gates` (or one row of constants for every token: a fixed decay a head); q, k, v are float rows; the state is float, lives in the request's slot and is
 // loaded before and stored after the item's rows, so prompts, portions and single tokens take the
 // same route and a position's sums are formed in the same order however the tokens were cut.
 //
@@ -70,7 +70,7 @@ template <int MODE, int KQ, bool VEC>
 __global__ __launch_bounds__(128) void state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
     int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ ga,
-    const float* __restrict__ gb, const float* __restrict__ skip, float* __restrict__ state, int64_t slot_stride,
+    const float* __restrict__ gb, int64_t gate_stride, const float* __restrict__ skip, float* __restrict__ state, int64_t slot_stride,
     const int* __restrict__ item_len, const int* __restrict__ item_tok_off, const int* __restrict__ item_slot,
     int heads, int qk_heads, int key_dim, int value_dim, int chunk) {
     extern __shared__ __attribute__((aligned(16))) float staged[];
@@ -89,8 +89,8 @@ __global__ __launch_bounds__(128) void state_scan_kernel(
     const float* qp = q + row0 * q_stride + (int64_t)qk_head * key_dim;
     const float* kp = k + row0 * k_stride + (int64_t)qk_head * key_dim;
     const float* vp = v + row0 * v_stride + (int64_t)head * value_dim + col0;
-    const float* ap = ga + row0 * heads + head;
-    const float* bp = gb + row0 * heads + head;
+    const float* ap = ga + row0 * gate_stride + head;
+    const float* bp = gb + row0 * gate_stride + head;
     float* op = out + row0 * ((int64_t)heads * value_dim) + (int64_t)head * value_dim + col0;
     const int nq = chunk * KW, nv = chunk * 16;
     const int total = 2 * nq + nv + 2 * chunk;          // floats of a staging buffer
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(128) void state_scan_kernel(
             float gate = 0.f;
             if (lane < 2 * chunk) {
                 const int r = lane < chunk ? lane : lane - chunk;
-                if (r < rows) gate = (lane < chunk ? ap : bp)[(int64_t)(t0 + r) * heads];
+                if (r < rows) gate = (lane < chunk ? ap : bp)[(int64_t)(t0 + r) * gate_stride];
             }
             for (int base = 0; base < totalv; base += 64 * NB) {
                 float4 x[NB];
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(128) void state_scan_kernel(
                     } else if (idx < total) {
                         const int j = idx - 2 * nq - nv;
                         const int r = j < chunk ? j : j - chunk;
-                        if (r < rows) src = (j < chunk ? ap : bp) + (int64_t)(t0 + r) * heads;
+                        if (r < rows) src = (j < chunk ? ap : bp) + (int64_t)(t0 + r) * gate_stride;
                     }
                     x[u] = src ? *src : 0.f;
                 }
@@ -319,13 +319,14 @@ extern "C" int st_unit_norm(float* x, int64_t stride, int num_tokens, int heads,
 
 extern "C" int st_state_scan(float* out, const float* q, int64_t q_stride, const float* k, int64_t k_stride,
                              const float* v, int64_t v_stride, const float* gate_a, const float* gate_b,
-                             const float* skip, float* state, int64_t slot_stride, const int* item_len,
+                             int64_t gate_stride, const float* skip, float* state, int64_t slot_stride, const int* item_len,
                              const int* item_tok_off, const int* item_slot, int num_items, int max_item_rows, int heads,
                              int qk_heads, int key_dim, int value_dim, int mode, hipStream_t stream) {
     ST_CHECK(num_items >= 0 && heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && key_dim > 0 && value_dim > 0,
              "state_scan: bad sizes");
     ST_CHECK(key_dim <= kScanMaxKeys, "state_scan: up to %d key channels a head, not %d", kScanMaxKeys, key_dim);
     ST_CHECK(mode == 0 || mode == 1, "state_scan: mode 0 (additive) or 1 (delta rule)");
+    ST_CHECK(gate_stride == 0 || gate_stride >= heads, "state_scan: gate rows overlap");
     ST_CHECK(num_items <= 65535 && (value_dim + 15) / 16 <= 65535, "state_scan: too many items or value channels");
     if (num_items == 0) return 0;
     ST_CHECK(out && q && k && v && gate_a && gate_b && state && item_len && item_tok_off && item_slot,
@@ -344,7 +345,7 @@ extern "C" int st_state_scan(float* out, const float* q, int64_t q_stride, const
                      v_stride % 4 == 0 && (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0;
 #define ST_SCAN(MODE, KQ, VEC)                                                                                      \
     state_scan_kernel<MODE, KQ, VEC><<<grid, 128, lds, stream>>>(out, q, q_stride, k, k_stride, v, v_stride, gate_a, \
-        gate_b, skip, state, slot_stride, item_len, item_tok_off, item_slot, heads, qk_heads, key_dim,              \
+        gate_b, gate_stride, skip, state, slot_stride, item_len, item_tok_off, item_slot, heads, qk_heads, key_dim,              \
         value_dim, chunk)
 #define ST_SCAN_MODE(KQ) do { if (mode == 0) { if (vec) ST_SCAN(0, KQ, true); else ST_SCAN(0, KQ, false); }        \
                               else { if (vec) ST_SCAN(1, KQ, true); else ST_SCAN(1, KQ, false); } } while (0)

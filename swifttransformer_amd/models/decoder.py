@@ -27,10 +27,13 @@ class Layer:
     ffn_norm: object
     feed_forward: object
     mixer_conv: object = None
+    mixer_out_norm: object = None
+    ffn_out_norm: object = None
+    side_input: object = None
 
     def parts(self):
-        return tuple(p for p in (self.mixer_norm, self.mixer_conv, self.mixer, self.ffn_norm, self.feed_forward)
-                     if p is not None)
+        return tuple(p for p in (self.mixer_norm, self.mixer_conv, self.mixer, self.mixer_out_norm, self.ffn_norm,
+                                 self.feed_forward, self.ffn_out_norm, self.side_input) if p is not None)
 
 
 def conv_cache_id(run: int):
@@ -60,7 +63,10 @@ class DecoderModel:
                 mixer=build_part("mixer", ls.mixer, H, dtype),
                 ffn_norm=opt("norm", ls.ffn_norm),
                 feed_forward=opt("feed_forward", ls.feed_forward),
-                mixer_conv=opt("token_conv", getattr(ls, "mixer_conv", None)))
+                mixer_conv=opt("token_conv", getattr(ls, "mixer_conv", None)),
+                mixer_out_norm=opt("norm", getattr(ls, "mixer_out_norm", None)),
+                ffn_out_norm=opt("norm", getattr(ls, "ffn_out_norm", None)),
+                side_input=opt("side_input", getattr(ls, "side_input", None)))
             needs = getattr(layer.arrangement, "needs", ())
             missing = [n for n in needs if getattr(layer, n) is None]
             if missing:
@@ -114,6 +120,13 @@ class DecoderModel:
             layer = self.layers[e.layer]
             if layer.mixer_conv is not None:
                 needs[conv_cache_id(run)] = layer.mixer_conv.cache_need()
+            if hasattr(layer.mixer, "cache_parts"):
+                # a mixer of several caches: each under (the run's cache id, the mixer's name for it)
+                if not e.write:
+                    raise ValueError(f"layer {e.layer}: a mixer with several caches has no read-only run")
+                for name, part_need in layer.mixer.cache_parts().items():
+                    needs[(e.cache, name)] = part_need
+                continue
             need = layer.mixer.cache_need()
             if need is None:
                 continue
@@ -161,11 +174,15 @@ class DecoderModel:
             K.arena.next_bank()      # what this run of a layer makes may be read until the next one ends
             if e.enter is not None:
                 x32 = self.entries[e.enter].forward(x32, first32, ctx)
+            if hasattr(layer.mixer, "cache_parts"):
+                cache = {name: caches.get((e.cache, name)) for name in layer.mixer.cache_parts()}
+            else:
+                cache = caches.get(e.cache)
             if layer.mixer_conv is not None:
-                x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write,
+                x32 = layer.arrangement.forward(x32, layer, ctx, cache, e.write,
                                                 conv_cache=caches.get(conv_cache_id(run)))
             else:
-                x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write)
+                x32 = layer.arrangement.forward(x32, layer, ctx, cache, e.write)
         return x32
 
     def forward_head(self, x32: torch.Tensor, ctx, want_rows: Optional[torch.Tensor] = None,

@@ -69,8 +69,8 @@ def _lib():
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_token_conv_state.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_int, _c_int,
                                             _c_int, _c_p]
-        lib.st_rotary.argtypes = [_c_p, _c_i64, _c_int, _c_p, _c_i64, _c_int, _c_int, _c_int, _c_p, _c_f, _c_p, _c_int,
-                                  _c_int, _c_p]
+        lib.st_rotary.argtypes = [_c_p, _c_i64, _c_int, _c_p, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p, _c_f,
+                                  _c_p, _c_int, _c_int, _c_p]
         lib.st_paged_write.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int,
                                        _c_int, _c_int, _c_f, _c_int, _c_p]
         lib.st_concat_cast.argtypes = [_c_p, _c_p, _c_int, _c_p, _c_int, _c_int, _c_int, _c_p]
@@ -78,10 +78,10 @@ def _lib():
         lib.st_sink_attention_lds.argtypes = [_c_int, _c_int, _c_int]
         lib.st_sink_attention.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p,
                                           _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int,
-                                          _c_int, _c_int, _c_int, _c_p]
+                                          _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_recurrence_gates.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
         lib.st_unit_norm.argtypes = [_c_p, _c_i64, _c_int, _c_int, _c_int, _c_f, _c_f, _c_p]
-        lib.st_state_scan.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_i64,
+        lib.st_state_scan.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
                                       _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_gated_group_norm.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                             _c_f, _c_int, _c_p]
@@ -91,14 +91,17 @@ def _lib():
         lib.st_gated_head_norm.argtypes = [_c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int,
                                            _c_f, _c_int, _c_p]
         lib.st_latent_write.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
-                                        _c_int, _c_int, _c_f, _c_int, _c_p]
-        lib.st_moe_route.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+                                        _c_int, _c_int, _c_f, _c_int, _c_p, _c_int, _c_p]
+        lib.st_moe_route.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_moe_align.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_moe_up.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                  _c_f, _c_int, _c_p]
+                                  _c_f, _c_int, _c_int, _c_p]
         lib.st_moe_down.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                     _c_f, _c_int, _c_p]
-        lib.st_moe_combine.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_f, _c_p]
+        lib.st_moe_combine.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_f, _c_p]
+        lib.st_dynamic_tanh.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_unit_add.argtypes = [_c_p, _c_p, _c_p, _c_int, _c_int, _c_f, _c_p]
+        lib.st_row_add.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
         _configured = True
@@ -359,7 +362,7 @@ def wide_offered(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
 # functions of the products' epilogues and of ``activation_multiply``, by the C interface's number
 # (csrc/activation.h; the names config files use for them)
 ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3, "gelu": 4, "gelu_erf": 4,
-               "relu_squared": 5, "relu2": 5}
+               "relu_squared": 5, "relu2": 5, "sigmoid": 6}
 
 
 def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_f32=False, algo=0,
@@ -798,12 +801,14 @@ def token_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx_a
 # ------------------------------------------- rotary positions, one-pool page write
 @_timed("rotary", lambda q, k, *a, **kw: {"rows": q.shape[0], "width": q.shape[1] + k.shape[1],
                                           "bytes": 2 * q.shape[0] * (q.shape[1] + k.shape[1]) * q.element_size()})
-def rotary(q: torch.Tensor, k: torch.Tensor, head_dim: int, freq: torch.Tensor, mult: float,
-           positions: torch.Tensor) -> None:
-    """In place on q [T, heads * head_dim] and k [T, kv_heads * head_dim] (dense rows, any row stride): of
-    every head the first 2 * len(freq) coordinates are turned, coordinate i paired with i + len(freq), by
-    the angle positions[t] * freq[i]; cosine and sine are multiplied by ``mult``.  Rows with a negative
-    position are left alone."""
+def rotary(q: torch.Tensor, k: Optional[torch.Tensor], head_dim: int, freq: torch.Tensor, mult: float,
+           positions: torch.Tensor, offset: int = 0, interleaved: bool = False) -> None:
+    """In place on q [T, heads * head_dim] and k [T, kv_heads * head_dim] (dense rows, any row stride; k may
+    be None): of every head the 2 * len(freq) coordinates from ``offset`` on are turned, coordinate i paired
+    with i + len(freq) (``interleaved``: 2i with 2i + 1), by the angle positions[t] * freq[i]; cosine and
+    sine are multiplied by ``mult``.  Rows with a negative position are left alone."""
+    if k is None:
+        k = q[:, :0]
     T = q.shape[0]
     half = freq.shape[0]
     _need(freq, "freq", torch.float32, (half,))
@@ -812,11 +817,11 @@ def rotary(q: torch.Tensor, k: torch.Tensor, head_dim: int, freq: torch.Tensor, 
         _need(t, name, q.dtype, (T, t.shape[1]), contiguous=False)
         if t.stride(1) != 1 or t.shape[1] % head_dim:
             raise KernelError(f"{name}: dense rows of whole heads")
-    if 2 * half > head_dim:
-        raise KernelError(f"{2 * half} turned coordinates do not fit a head of {head_dim}")
-    _check(_lib().st_rotary(_ptr(q), q.stride(0), q.shape[1] // head_dim, _ptr(k), k.stride(0), k.shape[1] // head_dim,
-                            head_dim, 2 * half, _ptr(freq), float(mult), _ptr(positions), T, dtype_code(q.dtype),
-                            _stream()))
+    if offset < 0 or offset + 2 * half > head_dim:
+        raise KernelError(f"{2 * half} turned coordinates from {offset} on do not fit a head of {head_dim}")
+    _check(_lib().st_rotary(_ptr(q), q.stride(0), q.shape[1] // head_dim, _ptr(k) if k.shape[1] else None, k.stride(0),
+                            k.shape[1] // head_dim, head_dim, 2 * half, int(offset), int(bool(interleaved)), _ptr(freq),
+                            float(mult), _ptr(positions), T, dtype_code(q.dtype), _stream()))
 
 
 @_timed("paged_write", lambda cache, src, *a, **kw: {"rows": src.shape[0], "width": src.shape[1],
@@ -871,9 +876,9 @@ def _d_sink_attention(q, k_cache, v_cache, token_item, positions, block_table, h
 def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, token_item: torch.Tensor,
                    positions: torch.Tensor, block_table: torch.Tensor, heads: int, scale: float, *,
                    window: int = 0, sink: bool = True, head_mix: Optional[torch.Tensor] = None,
-                   num_splits: int = 1, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   num_splits: int = 1, out: Optional[torch.Tensor] = None, keep_first: int = 0) -> torch.Tensor:
     """Each query row attends over its request's cached keys [max(0, p - window + 1), p] (window 0: from
-    0).  Every head's scaled products with a key are mixed over the heads by ``head_mix`` (float
+    0) and, with ``keep_first`` > 0, over the keys at positions below ``keep_first`` as well.  Every head's scaled products with a key are mixed over the heads by ``head_mix`` (float
     [heads, heads], row = receiving head; None: no mix) before the softmax; ``sink``: one is added to the
     softmax's denominator.
 
@@ -904,7 +909,8 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     _check(_lib().st_sink_attention(_ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), q.stride(0), _ptr(k_cache),
                                     k_cache.stride(0), _ptr(v_cache), v_cache.stride(0), _ptr(head_mix),
                                     _ptr(token_item), _ptr(positions), _ptr(block_table), block_table.shape[1], ps, T,
-                                    heads, nkv, dk, dv, float(scale), int(window), int(bool(sink)), int(num_splits),
+                                    heads, nkv, dk, dv, float(scale), int(window), int(keep_first), int(bool(sink)),
+                                    int(num_splits),
                                     dtype_code(q.dtype), _stream()))
     return out
 
@@ -978,8 +984,13 @@ def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate_a: torch.
         _need(t, name, torch.float32, (T, t.shape[1]), contiguous=False)
         if t.stride(1) != 1:
             raise KernelError(f"{name}: rows must be dense")
-    _need(gate_a, "gate_a", torch.float32, (T, heads))
-    _need(gate_b, "gate_b", torch.float32, (T, heads))
+    # one row of gates serves every token (constants a head), or a row a token
+    gate_rows = gate_a.shape[0]
+    if gate_rows not in (1, T) and T > 0:
+        raise KernelError(f"state_scan: gates for 1 or {T} rows, not {gate_rows}")
+    _need(gate_a, "gate_a", torch.float32, (gate_rows, heads))
+    _need(gate_b, "gate_b", torch.float32, (gate_rows, heads))
+    gate_stride = 0 if gate_rows == 1 else heads
     if skip is not None:
         _need(skip, "skip", torch.float32, (heads,))
     slot_stride = _slot_rows(state, "state", heads * kd * vd)
@@ -988,7 +999,7 @@ def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate_a: torch.
         _need(t, name, torch.int32, (B,))
     out = empty((T, heads * vd), torch.float32, q.device)
     _check(_lib().st_state_scan(_ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
-                                _ptr(gate_a), _ptr(gate_b), _ptr(skip), _ptr(state), slot_stride, _ptr(item_len),
+                                _ptr(gate_a), _ptr(gate_b), gate_stride, _ptr(skip), _ptr(state), slot_stride, _ptr(item_len),
                                 _ptr(item_tok_off), _ptr(item_slot), B, int(max_item_rows) or T, heads, qk_heads, kd, vd,
                                 {"additive": 0, "delta": 1}[mode], _stream()))
     return out
@@ -1110,16 +1121,24 @@ def gated_head_norm(o, gate: torch.Tensor, gain: torch.Tensor, heads: int, eps: 
 @_timed("latent_write", lambda cache, x, *a, **k: {"rows": x.shape[0], "width": x.shape[1],
                                                    "bytes": x.numel() * (4 + cache.element_size())})
 def latent_write(cache: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, token_item: torch.Tensor,
-                 positions: torch.Tensor, block_table: torch.Tensor) -> None:
-    """Each row of x (float [T, rank], dense rows of any stride) is normalised to unit root mean
-    square, multiplied by ``gain`` and stored as its token's entry of ``cache``
-    [pages, 1, page_size, entry] with entry >= rank (the rest of an entry is cleared)."""
+                 positions: torch.Tensor, block_table: torch.Tensor, tail: int = 0,
+                 tail_freq: Optional[torch.Tensor] = None) -> None:
+    """Each row of x (float [T, rank + tail], dense rows of any stride): its first ``rank`` values are
+    normalised to unit root mean square, multiplied by ``gain`` and stored as its token's entry of ``cache``
+    [pages, 1, page_size, entry] with entry >= rank + tail; the ``tail`` values after them follow in the
+    entry as they are, or, with ``tail_freq`` (float [tail / 2]), turned by the token's position (pairs
+    2i, 2i + 1; angle position * tail_freq[i]); the rest of an entry is cleared."""
     num_pages, one, ps, entry = cache.shape
-    T, rank = x.shape
+    T = x.shape[0]
+    rank = x.shape[1] - int(tail)
     _need(cache, "cache", None, (num_pages, 1, ps, entry), contiguous=False)
-    if cache.stride()[1:] != (ps * entry, entry, 1) or entry < rank:
-        raise KernelError("latent_write: pages of one head must be contiguous and an entry as wide as the rank")
-    _need(x, "x", torch.float32, (T, rank), contiguous=False)
+    if rank <= 0 or cache.stride()[1:] != (ps * entry, entry, 1) or entry < rank + tail:
+        raise KernelError("latent_write: pages of one head must be contiguous and an entry as wide as the row")
+    if tail_freq is not None:
+        _need(tail_freq, "tail_freq", torch.float32, (tail // 2,))
+        if tail % 2:
+            raise KernelError("latent_write: a turned tail has an even size")
+    _need(x, "x", torch.float32, (T, rank + tail), contiguous=False)
     if x.stride(1) != 1:
         raise KernelError("x: rows must be dense")
     _need(gain, "gain", torch.float32, (rank,))
@@ -1128,7 +1147,7 @@ def latent_write(cache: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: 
     _need(block_table, "block_table", torch.int32)
     _check(_lib().st_latent_write(_ptr(cache), cache.stride(0), _ptr(x), x.stride(0), _ptr(gain), _ptr(token_item),
                                   _ptr(positions), _ptr(block_table), block_table.shape[1], ps, T, rank, entry,
-                                  float(eps), dtype_code(cache.dtype), _stream()))
+                                  float(eps), int(tail), _ptr(tail_freq), dtype_code(cache.dtype), _stream()))
 
 
 # ---------------------------------------------------------------- routed experts
@@ -1145,7 +1164,7 @@ def moe_capacity(num_tokens: int, top: int, experts: int, tile: int) -> int:
     return -(-num_tokens * top // tile) * tile + tile * experts
 
 
-def _d_moe(x, logits, w_gate, w_up, w_down, residual, *, top, limit, out_scale=1.0, token_item=None):
+def _d_moe(x, logits, w_gate, w_up, w_down, residual, *, top, limit=0.0, out_scale=1.0, token_item=None, **kw):
     T, W = x.shape
     E, F, _ = w_gate.shape
     used = min(E, T * top)
@@ -1155,12 +1174,17 @@ def _d_moe(x, logits, w_gate, w_up, w_down, residual, *, top, limit, out_scale=1
 
 @_timed("routed_experts", _d_moe)
 def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
-                   w_down: torch.Tensor, residual: torch.Tensor, *, top: int, limit: float, out_scale: float = 1.0,
-                   token_item: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   w_down: torch.Tensor, residual: Optional[torch.Tensor], *, top: int, limit: float = 0.0,
+                   out_scale: float = 1.0, token_item: Optional[torch.Tensor] = None,
+                   style: str = "scaled_input") -> torch.Tensor:
     """residual <- residual + out_scale * sum over a row's ``top`` best experts e (by ``logits``) of
     Wd[e] y with y = g * sigmoid(1.702 g) * (u + 1), g = min(s * Wg[e] x, limit),
     u = clamp(s * Wu[e] x, -limit, limit), s = sigmoid(logit of e).  In place on ``residual``
     (float [T, width]), which is returned.
+
+    ``style`` "softmax_output": the weights of a row's experts are the softmax over their logits alone and
+    multiply the experts' results, sum_e s_e Wd[e] (silu(Wg[e] x) * (Wu[e] x)), with no limit.  Then
+    ``residual`` may be None: the weighted sum itself is returned (a new float tensor).
 
     x: [T, width]; logits: float [T, experts]; w_gate, w_up: [experts, inner, width]; w_down:
     [experts, width, inner].  Rows whose ``token_item`` is negative are left as they are."""
@@ -1171,7 +1195,13 @@ def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, 
     _need(w_gate, "w_gate", None, (E, F, W))
     _need(w_up, "w_up", w_gate.dtype, (E, F, W))
     _need(w_down, "w_down", w_gate.dtype, (E, W, F))
-    _need(residual, "residual", torch.float32, (T, W))
+    if style not in ("scaled_input", "softmax_output"):
+        raise KernelError(f"routed_experts: unknown style {style!r}")
+    on_output = style == "softmax_output"
+    if residual is None and not on_output:
+        raise KernelError("routed_experts: this style adds to a residual stream")
+    if residual is not None:
+        _need(residual, "residual", torch.float32, (T, W))
     if token_item is not None:
         _need(token_item, "token_item", torch.int32, (T,))
     lib, dev, code, st = _lib(), x.device, dtype_code(x.dtype), _stream()
@@ -1183,10 +1213,18 @@ def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, 
     place = empty((T * top,), torch.int32, dev)
     tile_expert = empty((cap // tile,), torch.int32, dev)
     y = empty((cap, F), x.dtype, dev)
-    _check(lib.st_moe_route(_ptr(ids), _ptr(wts), _ptr(logits), _ptr(token_item), T, E, int(top), st))
+    _check(lib.st_moe_route(_ptr(ids), _ptr(wts), _ptr(logits), _ptr(token_item), T, E, int(top), int(on_output), st))
     _check(lib.st_moe_align(_ptr(sorted_pairs), _ptr(place), _ptr(tile_expert), _ptr(ids), T * top, E, cap, tile, st))
     _check(lib.st_moe_up(_ptr(y), _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(sorted_pairs), _ptr(tile_expert),
-                         _ptr(wts), cap, tile, int(top), W, F, float(limit), code, st))
+                         _ptr(wts), cap, tile, int(top), W, F, float(limit), int(on_output), code, st))
+    if on_output:
+        out = residual if residual is not None else empty((T, W), torch.float32, dev)
+        pair_out = empty((cap, W), torch.float32, dev)
+        _check(lib.st_moe_down(None, None, _ptr(pair_out), _ptr(y), _ptr(w_down), _ptr(sorted_pairs),
+                               _ptr(tile_expert), cap, tile, int(top), W, F, 1.0, code, st))
+        _check(lib.st_moe_combine(_ptr(out), _ptr(residual), _ptr(pair_out), _ptr(place), _ptr(wts), T, int(top), W,
+                                  float(out_scale), st))
+        return out
     if top == 1:
         _check(lib.st_moe_down(_ptr(residual), _ptr(residual), None, _ptr(y), _ptr(w_down), _ptr(sorted_pairs),
                                _ptr(tile_expert), cap, tile, 1, W, F, float(out_scale), code, st))
@@ -1194,9 +1232,65 @@ def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, 
         pair_out = empty((cap, W), torch.float32, dev)
         _check(lib.st_moe_down(None, None, _ptr(pair_out), _ptr(y), _ptr(w_down), _ptr(sorted_pairs),
                                _ptr(tile_expert), cap, tile, int(top), W, F, float(out_scale), code, st))
-        _check(lib.st_moe_combine(_ptr(residual), _ptr(residual), _ptr(pair_out), _ptr(place), T, int(top), W,
+        _check(lib.st_moe_combine(_ptr(residual), _ptr(residual), _ptr(pair_out), _ptr(place), None, T, int(top), W,
                                   float(out_scale), st))
     return residual
+
+
+# -------------------------------------------- float operations on the residual stream
+@_timed("dynamic_tanh", lambda x, *a, **k: {"rows": (k.get("rows").shape[0] if k.get("rows") is not None else x.shape[0]),
+                                            "width": x.shape[1], "bytes": 10 * x.shape[1] *
+                                            (k.get("rows").shape[0] if k.get("rows") is not None else x.shape[0])})
+def dynamic_tanh(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], alpha: torch.Tensor, *,
+                 rows: Optional[torch.Tensor] = None, out_t: Optional[torch.Tensor] = None,
+                 out_f32: Optional[torch.Tensor] = None, base: Optional[torch.Tensor] = None) -> None:
+    """y = tanh(alpha * x) * weight + bias per element of the float rows x [T, width] (of the rows picked by
+    ``rows``, int32, negative entries skipped); ``alpha``: float [1] on the device.  ``base`` (float, the
+    result's shape): y += base.  Written to ``out_f32`` (float) and / or ``out_t`` (float or bfloat16)."""
+    T, W = x.shape
+    n = rows.shape[0] if rows is not None else T
+    _need(x, "x", torch.float32, (T, W))
+    _need(weight, "weight", torch.float32, (W,))
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (W,))
+    _need(alpha, "alpha", torch.float32, (1,))
+    if rows is not None:
+        _need(rows, "rows", torch.int32, (n,))
+    if out_t is None and out_f32 is None:
+        raise KernelError("dynamic_tanh: no output")
+    if out_f32 is not None:
+        _need(out_f32, "out_f32", torch.float32, (n, W))
+    if out_t is not None:
+        _need(out_t, "out_t", None, (n, W))
+    if base is not None:
+        _need(base, "base", torch.float32, (n, W))
+    _check(_lib().st_dynamic_tanh(_ptr(out_t), _ptr(out_f32), _ptr(x), _ptr(rows), _ptr(weight), _ptr(bias), _ptr(alpha),
+                                  _ptr(base), n, W, dtype_code(out_t.dtype) if out_t is not None else F32, _stream()))
+
+
+@_timed("unit_add", lambda x, y, *a, **k: {"rows": x.shape[0], "width": x.shape[1], "bytes": 12 * x.numel()})
+def unit_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """x += y / sqrt(mean(y^2) + eps) * weight row by row, in place on the float rows x [T, width]."""
+    T, W = x.shape
+    _need(x, "x", torch.float32, (T, W))
+    _need(y, "y", torch.float32, (T, W))
+    _need(weight, "weight", torch.float32, (W,))
+    _check(_lib().st_unit_add(_ptr(x), _ptr(y), _ptr(weight), T, W, float(eps), _stream()))
+    return x
+
+
+@_timed("row_add", lambda x, *a, **k: {"rows": x.shape[0], "width": x.shape[1], "bytes": 12 * x.numel()})
+def row_add(x: torch.Tensor, first: Optional[torch.Tensor], vec: torch.Tensor) -> torch.Tensor:
+    """x (+ first) + vec: float rows [T, width], a second stream of the same shape or None, and one float
+    vector [width] for every row.  Returns a new tensor."""
+    T, W = x.shape
+    _need(x, "x", torch.float32, (T, W))
+    if first is not None:
+        _need(first, "first", torch.float32, (T, W))
+    _need(vec, "vec", torch.float32, (W,))
+    out = empty((T, W), torch.float32, x.device)
+    _check(_lib().st_row_add(_ptr(out), _ptr(x), _ptr(first), _ptr(vec), T, W, _stream()))
+    return out
 
 
 def probe_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, pattern: int = 0) -> None:

@@ -6,6 +6,9 @@ pre-norm (reference src/csrc/model/gpt/gpt.cc:325-335, :347-391, :423-436, :467-
     half; a factor on the branches is the mixer's and the feed-forward's own parameter)
 post-norm (the reference refuses it, gpt.cc:238-240):
     r = N1(x + Mix(x)); x' = N2(r + FFN(r))
+sandwich (norms before and after each sublayer; the reference has no such block):
+    r = x + N1b(Mix(N1(x))); s = r + N2b(FFN(N2(r))); x' = s + Side(s, token)
+    (the feed-forward and the side input are optional)
 The residual stream is float; parts that multiply matrices take the storage type."""
 from __future__ import annotations
 
@@ -61,3 +64,30 @@ class PostNorm(Part):
         u32 = layer.feed_forward.forward(r_t, r32, ctx)
         _, y32 = layer.ffn_norm.forward(u32, out_t=False, out_f32=True)
         return y32
+
+
+class Sandwich(Part):
+    """params: feed_forward (bool, default True).  The mixer and the feed-forward are asked for their
+    results alone (``residual32`` None, which they must allow: ``raw_output_ok``); the norm after each adds
+    its result to the stream (``forward_onto``).  A ``side_input`` part of the layer acts on the stream last."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        super().__init__(spec, hidden_size, dtype)
+        self.has_ffn = bool(spec.params.get("feed_forward", True))
+        self.needs = (("mixer_norm", "mixer_out_norm", "ffn_norm", "feed_forward", "ffn_out_norm") if self.has_ffn
+                      else ("mixer_norm", "mixer_out_norm"))
+
+    def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True) -> torch.Tensor:
+        for part in (layer.mixer, layer.feed_forward if self.has_ffn else None):
+            if part is not None and not getattr(part, "raw_output_ok", False):
+                raise ValueError(f"{type(part).__name__} cannot give its result without the residual stream")
+        a, _ = layer.mixer_norm.forward(x32, out_t=True)
+        m32 = layer.mixer.forward(a, None, ctx, cache, write)
+        x32 = layer.mixer_out_norm.forward_onto(m32, x32)
+        if self.has_ffn:
+            d, _ = layer.ffn_norm.forward(x32, out_t=True)
+            f32 = layer.feed_forward.forward(d, None, ctx)
+            x32 = layer.ffn_out_norm.forward_onto(f32, x32)
+        if layer.side_input is not None:
+            x32 = layer.side_input.forward(x32, ctx)
+        return x32

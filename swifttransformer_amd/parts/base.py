@@ -13,8 +13,12 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
   norm          ``forward(x32, out_t=bool, out_f32=bool, rows=None) -> (y_t, y32)``
   mixer         ``cache_need() -> CacheNeed | None``; ``use_position(position)``: the model's
                 position part, told once after construction;
-                ``forward(x_t, residual32, ctx, cache, write=True) -> x32`` (= residual + mix(x))
-  feed_forward  ``forward(x_t, residual32, ctx) -> x32`` (= residual + ffn(x))
+                ``forward(x_t, residual32, ctx, cache, write=True) -> x32`` (= residual + mix(x));
+                ``residual32`` None where the mixer sets ``raw_output_ok``: the float mix(x) alone.
+                A mixer that keeps several caches offers ``cache_parts() -> {name: CacheNeed}``
+                instead of ``cache_need`` and gets ``cache`` as a dict name -> view
+  feed_forward  ``forward(x_t, residual32, ctx) -> x32`` (= residual + ffn(x)); ``residual32`` None
+                where it sets ``raw_output_ok``: the float ffn(x) alone
   position      ``embedding_addend(ctx)`` rows to add to the token embedding, or None;
                 ``rotates`` (bool) and ``rotate(q, k, ctx)``: in-place change of the step's queries
                 [T, heads*head_dim] and keys [T, kv_heads*head_dim] (views of the mixer's QKV
@@ -28,6 +32,8 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
                 that has a ``mixer_conv`` part)
   token_conv    ``cache_need() -> CacheNeed``; ``forward(y32, ctx, cache) -> y_t``: a short causal
                 filter over time on what a mixer reads, with its last inputs as per-request state
+  side_input    ``forward(x32, ctx) -> x32``: what a layer adds to the stream after its feed-forward
+                from an input of the token's own (a per-layer token embedding)
   reentry       ``forward(x32, first32, ctx) -> x32``: what happens to the residual stream before a run
                 of a layer that the schedule marks (``ScheduleEntry.enter``); ``first32`` is the
                 embedding's output of the step
@@ -52,7 +58,7 @@ from ..weights.loader import TensorSpec
 from .spec import PartSpec
 
 CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "arrangement", "token_conv",
-              "reentry")
+              "reentry", "side_input")
 _REGISTRY: Dict[str, Dict[str, Callable]] = {c: {} for c in CATEGORIES}
 
 
@@ -80,7 +86,8 @@ class CacheNeed:
     per token each; ``window`` > 0 means only the last ``window`` tokens are ever
     read, so pages behind it are given back.  ``values`` False: one vector per token serves as
     key and as value (a latent cache); no second pool is allocated and the view's ``v`` is its ``k``.
-    ``value_dim`` > 0: the values' heads have that size instead of ``head_dim``.
+    ``value_dim`` > 0: the values' heads have that size instead of ``head_dim``.  ``keep_first`` > 0 (with a
+    window): the first ``keep_first`` tokens are read for ever, so their pages are never given back.
     kind "state": a fixed-size tensor per request (``state_shape``, ``state_dtype``),
     living in the request's state slot."""
     kind: str
@@ -91,10 +98,11 @@ class CacheNeed:
     state_dtype: Optional[torch.dtype] = None
     values: bool = True
     value_dim: int = 0
+    keep_first: int = 0
 
     def group_key(self):
         return (self.kind, self.num_kv_heads, self.head_dim, self.window, self.state_shape,
-                self.state_dtype, self.values, self.value_dim)
+                self.state_dtype, self.values, self.value_dim, self.keep_first)
 
 
 @dataclass

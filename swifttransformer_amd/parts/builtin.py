@@ -1,18 +1,22 @@
 """Registration of the parts that ship with the engine."""
 from .base import register_part
-from .norm import LayerNorm
+from .norm import LayerNorm, DynamicTanh
 from .position import LearnedPositions, NoPositions, RotaryPositions
 from .embedding import TokenEmbedding, LMHead
 from .feed_forward import DenseFeedForward
 from .attention import PagedAttention
-from .arrangement import PreNorm, PostNorm
+from .arrangement import PreNorm, PostNorm, Sandwich
 from .conv import CausalTokenConv
 from .linear_attention import GatedLinearAttention
 from .latent_attention import LatentAttention
 from .routed import RoutedExperts
 from .sink_attention import SinkAttention
 from .state_space import Mamba2Mixer, GatedDeltaRule
-from .reentry import InputInjection
+from .reentry import InputInjection, AdditiveEntry
+from .window_attention import GatedWindowAttention
+from .retention import Retention
+from .parallel import ParallelMixers
+from .side_input import TokenSideInput
 
 register_part("norm", "layer_norm", LayerNorm)
 register_part("position", "learned", LearnedPositions)
@@ -32,3 +36,10 @@ register_part("mixer", "sink_attention", SinkAttention)
 register_part("mixer", "mamba2", Mamba2Mixer)
 register_part("mixer", "gated_delta", GatedDeltaRule)
 register_part("reentry", "input_injection", InputInjection)
+register_part("norm", "dynamic_tanh", DynamicTanh)
+register_part("arrangement", "sandwich", Sandwich)
+register_part("reentry", "additive", AdditiveEntry)
+register_part("mixer", "gated_window_attention", GatedWindowAttention)
+register_part("mixer", "retention", Retention)
+register_part("mixer", "parallel", ParallelMixers)
+register_part("side_input", "token_side", TokenSideInput)

@@ -6,7 +6,12 @@ the two sums in float and normalises in the storage type; here the whole
 computation is in float on the float residual stream, with the variance taken
 from centred values.  The parameter ``center`` = False gives the form that takes no mean
 off, y = x * rsqrt(mean(x^2) + eps) * gamma (+ beta) (reference src/csrc/kernel/rmsnorm.cu):
-the same kernels and the same fusion into a product, by a flag."""
+the same kernels and the same fusion into a product, by a flag.
+
+``DynamicTanh`` is a norm that takes no statistics of the row at all: y = tanh(alpha x) * w + b per
+element, alpha one learned number.  It can also add its result to a stream on the way
+(``forward_onto``), which is how a branch's result is normalised as it enters the residual stream.
+The reference has no such part."""
 from __future__ import annotations
 
 from typing import Dict, List, Optional, Tuple
@@ -69,3 +74,45 @@ class LayerNorm(Part):
             return y32, y32
         K.layernorm(x32, self.gamma, self.beta, self.eps, rows=rows, out_t=yt, out_f32=y32, center=self.center)
         return yt, y32
+
+
+class DynamicTanh(Part):
+    """params: width (int, default hidden_size), bias (bool, default True).  names: weight, bias, alpha
+    (a tensor of no dimensions)."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        super().__init__(spec, hidden_size, dtype)
+        self.width = int(self.param("width", hidden_size))
+        self.has_bias = bool(spec.params.get("bias", True))
+        self.gamma = self.beta = self.alpha = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [TensorSpec(self.name("weight"), (self.width,), "vector", init="gain"),
+                 TensorSpec(self.name("alpha"), (), "vector", init="gain")]
+        if self.has_bias:
+            specs.append(TensorSpec(self.name("bias"), (self.width,), "vector"))
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.gamma = tensors[self.name("weight")]
+        self.alpha = tensors[self.name("alpha")].reshape(1).contiguous()
+        self.beta = tensors[self.name("bias")] if self.has_bias else None
+
+    def forward(self, x32: torch.Tensor, *, out_t: bool = True, out_f32: bool = False,
+                rows: Optional[torch.Tensor] = None) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+        n = rows.shape[0] if rows is not None else x32.shape[0]
+        if self.dtype == torch.float32 and out_t and out_f32:
+            out_t = False                                   # one float result serves as both
+            both = True
+        else:
+            both = False
+        yt = K.empty((n, self.width), self.dtype, x32.device) if out_t else None
+        y32 = K.empty((n, self.width), torch.float32, x32.device) if out_f32 else None
+        K.dynamic_tanh(x32, self.gamma, self.beta, self.alpha, rows=rows, out_t=yt, out_f32=y32)
+        return (y32, y32) if both else (yt, y32)
+
+    def forward_onto(self, y32: torch.Tensor, stream32: torch.Tensor) -> torch.Tensor:
+        """stream32 + norm(y32), float, a new tensor."""
+        out = K.empty(tuple(stream32.shape), torch.float32, stream32.device)
+        K.dynamic_tanh(y32, self.gamma, self.beta, self.alpha, out_f32=out, base=stream32)
+        return out

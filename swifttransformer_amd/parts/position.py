@@ -55,11 +55,29 @@ def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None):
     are blended between f_i (pairs that turn more than ``fast`` times within ``original`` positions keep
     theirs) and f_i / factor (pairs that turn fewer than ``slow`` times), linearly in the pair's index
     between the two border indices d(fast) and d(slow), d(t) = dims ln(original / (2 pi t)) / (2 ln base);
-    cosine and sine are then multiplied by 0.1 ln(factor) + 1."""
+    cosine and sine are then multiplied by 0.1 ln(factor) + 1.
+    With ``scaling`` = {factor, original, low, high} the rule goes by a pair's wavelength l = 2 pi / f_i:
+    l < original / high keeps f_i, l > original / low takes f_i / factor, and between the two
+    s = (original / l - low) / (high - low) blends them, (1 - s) f_i / factor + s f_i; cosine and sine
+    keep their size."""
     half = dims // 2
     f = [float(base) ** (-2.0 * i / dims) for i in range(half)]
     if not scaling:
         return f, 1.0
+    if "low" in scaling and "high" in scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+        low, high = float(scaling["low"]), float(scaling["high"])
+        out = []
+        for fi in f:
+            wave = 2.0 * math.pi / fi
+            if wave < orig / high:
+                out.append(fi)
+            elif wave > orig / low:
+                out.append(fi / factor)
+            else:
+                s = (orig / wave - low) / (high - low)
+                out.append((1.0 - s) * fi / factor + s * fi)
+        return out, 1.0
     factor, orig = float(scaling["factor"]), float(scaling["original"])
     border = lambda turns: dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
     lo = max(math.floor(border(float(scaling["fast"]))), 0)
@@ -73,7 +91,8 @@ def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None):
 
 class RotaryPositions(PositionEncoding):
     """params: head_dim (int), dims (int, even, <= head_dim: the coordinates of a head that turn), base
-    (float), scaling (None, or {factor, original, fast, slow}).  It adds nothing to the embedding; mixers
+    (float), scaling (None, {factor, original, fast, slow} or {factor, original, low, high}: see
+    ``rotary_frequencies``), interleaved (bool, default False: pairs are 2i, 2i + 1 instead of i, i + dims / 2).  It adds nothing to the embedding; mixers
     call ``rotate`` on their queries and keys.  Positions, angles, cosine and sine are float."""
     rotates = True
 
@@ -83,6 +102,7 @@ class RotaryPositions(PositionEncoding):
         self.dims = int(self.param("dims"))
         if self.dims % 2 or not 0 < self.dims <= self.head_dim:
             raise ValueError(f"rotary dims must be even and at most the head size {self.head_dim}, got {self.dims}")
+        self.interleaved = bool(spec.params.get("interleaved", False))
         freq, self.mult = rotary_frequencies(self.dims, float(self.param("base")), spec.params.get("scaling"))
         self._freq_host = torch.tensor(freq, dtype=torch.float64).to(torch.float32)
         self.freq: Optional[torch.Tensor] = None
@@ -95,4 +115,4 @@ class RotaryPositions(PositionEncoding):
     def rotate(self, q, k, ctx) -> None:
         if self.freq is None or self.freq.device != q.device:
             self.freq = self._freq_host.to(q.device)
-        K.rotary(q, k, self.head_dim, self.freq, self.mult, ctx.positions)
+        K.rotary(q, k, self.head_dim, self.freq, self.mult, ctx.positions, interleaved=self.interleaved)

@@ -7,6 +7,11 @@ layers, chosen by a router.
     the token's result is the sum over its experts (the weights are not renormalised and multiply
     the expert's input, not its output)
 
+or, ``style`` "softmax_output":
+
+    z = Wr x + br (float);  the ``top`` largest z choose the experts;  s = softmax over the chosen z alone
+    expert e:  Wd (silu(Wg x) * (Wu x));  the token's result is sum_e s_e expert_e(x)
+
 Routing, sorting by expert and the experts' products all run on the device with launch shapes
 that depend on the number of rows only, so steps with this part are recorded like any other
 (``csrc/moe.hip``).  The reference has no such part."""
@@ -22,16 +27,21 @@ from .base import Part
 
 
 class RoutedExperts(Part):
-    """params: experts (int), top (int), inner (int: width inside an expert), limit (float),
-    residual_scale (float, default 1).  names: ``router`` and the patterns ``gate``, ``up``, ``down``
-    with ``{e}`` for the expert's number."""
+    """params: experts (int), top (int), inner (int: width inside an expert), limit (float, of the
+    "scaled_input" style), residual_scale (float, default 1), style ("scaled_input", the default, or
+    "softmax_output"), router_bias (bool, default False).  names: ``router`` (``router_bias``) and the
+    patterns ``gate``, ``up``, ``down`` with ``{e}`` for the expert's number."""
+
+    raw_output_ok = True     # with the "softmax_output" style, forward(..., residual32=None) returns the sum alone
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
         self.experts = int(self.param("experts"))
         self.top = int(self.param("top"))
         self.inner = int(self.param("inner"))
-        self.limit = float(self.param("limit"))
+        self.style = str(spec.params.get("style", "scaled_input"))
+        self.limit = float(self.param("limit")) if self.style == "scaled_input" else 0.0
+        self.router_bias = bool(spec.params.get("router_bias", False))
         self.residual_scale = float(spec.params.get("residual_scale", 1.0))
         if not 1 <= self.top <= min(self.experts, 16):
             raise ValueError(f"1 to 16 of {self.experts} experts a token, not {self.top}")
@@ -42,6 +52,8 @@ class RoutedExperts(Part):
     def tensor_specs(self) -> List[TensorSpec]:
         H, F = self.hidden_size, self.inner
         specs = [TensorSpec(self.name("router"), (self.experts, H), "matrix")]
+        if self.router_bias:
+            specs.append(TensorSpec(self.name("router_bias"), (self.experts,), "vector"))
         for e in range(self.experts):
             specs += [TensorSpec(self._expert("gate", e), (F, H), "matrix"),
                       TensorSpec(self._expert("up", e), (F, H), "matrix"),
@@ -50,10 +62,12 @@ class RoutedExperts(Part):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.w_router = tensors[self.name("router")]
+        self.b_router = tensors[self.name("router_bias")] if self.router_bias else None
         stack = lambda which: torch.stack([tensors[self._expert(which, e)] for e in range(self.experts)]).contiguous()
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
 
     def forward(self, x_t: torch.Tensor, residual32: torch.Tensor, ctx) -> torch.Tensor:
-        logits = K.gemm(x_t, self.w_router, out_f32=True)
+        logits = K.gemm(x_t, self.w_router, bias=self.b_router, out_f32=True)
         return K.routed_experts(x_t, logits, self.w_gate, self.w_up, self.w_down, residual32, top=self.top,
-                                limit=self.limit, out_scale=self.residual_scale, token_item=ctx.token_item)
+                                limit=self.limit, out_scale=self.residual_scale, token_item=ctx.token_item,
+                                style=self.style)

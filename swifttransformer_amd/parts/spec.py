@@ -25,6 +25,9 @@ class LayerSpec:
     ffn_norm: Optional[PartSpec]
     feed_forward: Optional[PartSpec]
     mixer_conv: Optional[PartSpec] = None   # a short filter over time on what the mixer reads
+    mixer_out_norm: Optional[PartSpec] = None   # a norm on the mixer's result before it enters the stream
+    ffn_out_norm: Optional[PartSpec] = None     # the same for the feed-forward's result
+    side_input: Optional[PartSpec] = None       # what the layer adds from an input of the token's own
 
 
 @dataclass
