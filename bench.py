@@ -208,8 +208,8 @@ def kernel_times(args) -> int:
     return 0
 
 
-def side_by_side(args, shape: str, other: str = "zitupel") -> int:
-    """Another architecture (Zitupel, Zimorax) beside OPT at the same layer sizes (width, heads, feed-forward width of OPT
+def side_by_side(args, shape: str, other: str = "zitupel", beside=("opt",)) -> int:
+    """Another architecture (Zitupel, Zimorax, Gisedra) beside OPT (``beside``: or other families) at the same layer sizes (width, heads, feed-forward width of OPT
     ``shape``; the same number of layers, 8 unless ``--layers`` says otherwise; random weights):
     decode tokens/s at batch 1, 8 and 64 from 1,024-token prompts, a 2,048-token prefill, and for
     both the per-kernel times of one decode step at batch ``--batch`` and of the prefill with their
@@ -226,7 +226,7 @@ def side_by_side(args, shape: str, other: str = "zitupel") -> int:
     dt = parse_dtype(args.dtype)
     batch = args.batch
     out = {"shape": shape, "layers": layers, "dtype": args.dtype, "models": {}}
-    for family in (other, "opt"):
+    for family in (other,) + tuple(beside):
         over = {"num_layers": layers} if family != "opt" else {"num_hidden_layers": layers}
         hp = hyper_param_by_name(f"{family}_{shape}", **over)
         model = random_model(hp, dt, 0, "cuda:0")
@@ -590,9 +590,11 @@ def main() -> int:
     ap.add_argument("--workload", default="decode-1.3b",
                     choices=["decode-1.3b", "mixed-6.7b", "mixed-1.3b", "ttft", "decode-30b", "decode-family",
                              "zitupel-125m", "zitupel-1.3b", "zitupel-6.7b",
-                             "zimorax-125m", "zimorax-1.3b", "zimorax-6.7b"],
+                             "zimorax-125m", "zimorax-1.3b", "zimorax-6.7b",
+                             "gisedra-125m", "gisedra-1.3b", "gisedra-6.7b"],
                     help="decode-1.3b is the default line; the others are the other model shapes; zitupel-<size>, "
-                         "zimorax-<size>: that architecture beside OPT at the same layer sizes")
+                         "zimorax-<size>: that architecture beside OPT at the same layer sizes; gisedra-<size>: "
+                         "Gisedra beside Zitupel and Zimorax (whose kernels are its kernels' likes) and OPT")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -618,6 +620,8 @@ def main() -> int:
     if args.workload.startswith(("zitupel-", "zimorax-")):
         family, shape = args.workload.split("-", 1)
         return side_by_side(args, shape, family)
+    if args.workload.startswith("gisedra-"):
+        return side_by_side(args, args.workload.split("-", 1)[1], "gisedra", beside=("zitupel", "zimorax", "opt"))
     steps = min(args.steps, CONTEXT - PROMPT_LEN)
     elem = 2 if args.dtype == "bf16" else 4
     biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)

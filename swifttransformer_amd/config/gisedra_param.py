@@ -128,8 +128,6 @@ class GisedraHyperParam:
                               f"{rank} + {r}")
         if r:
             _check_rot(m.get("rot"), f"{w}.rot", r, scaling_ok=True)
-            if m["rot"]["dims"] != r:
-                raise ConfigError(f"config.json: {w}.rot.dims must equal rot_dim ({r}), got {m['rot']['dims']}")
         if m.get("mask") is not None:
             _need(m["mask"], "size", f"{w}.mask", (int,), 1)
 

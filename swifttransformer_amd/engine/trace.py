@@ -33,10 +33,12 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
         raise ValueError(f"--dtype must be bfloat16 or float32, got {dtype!r}")
     os.makedirs(out_dir, exist_ok=True)
     model = load_model(model_dir, _DTYPES[dtype], device)
-    # the pool holds max_tokens tokens; a request's share is counted in whole pages
+    # the pool holds max_tokens tokens; a request's share is counted in whole pages.  No request is longer
+    # than what all live requests may hold together, so a block table need be no wider than the pool has
+    # pages, also where a windowed cache gives pages back and a table goes on past them
     num_pages = max(1, -(-max_tokens // page_size))
     runner = ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages,
-                                           max_seqs=max_live), device,
+                                           max_seqs=max_live, max_pages_per_seq=num_pages), device,
                          max_batched_tokens=min(max(max_tokens, 1), 4096))
     index: Dict[str, list] = {}
     try:

@@ -25,7 +25,8 @@ def _latent(hp: GisedraHyperParam, p: str, mx: dict) -> PartSpec:
     return PartSpec("latent_attention",
                     {"num_heads": mx["heads"], "key_dim": mx["dim"], "value_dim": mx["vdim"], "rank": mx["kv_rank"],
                      "scale": float(mx["scale"]), "eps": hp.norm_eps, "rot_dim": mx["rot_dim"],
-                     "rot_base": float(rot.get("base", 10000.0)), "rot_scaling": rot.get("scaling"),
+                     "rot_dims": int(rot.get("dims", mx["rot_dim"]) or 0), "rot_base": float(rot.get("base", 10000.0)),
+                     "rot_scaling": rot.get("scaling"),
                      "window": int((mx.get("mask") or {}).get("size", 0))},
                     {"q": f"{p}.q", "down": f"{p}.dkv", "down_norm": f"{p}.dkv.norm", "up_k": f"{p}.uk",
                      "up_v": f"{p}.uv", "out": f"{p}.o"})

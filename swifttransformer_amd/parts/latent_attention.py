@@ -37,8 +37,8 @@ class LatentAttention(PagedAttention):
     """params: num_heads, key_dim, value_dim, rank, scale (float), eps (float, of the latent's norm),
     own_latent (bool, default True; False: the layer reads another layer's cache and has no
     down-projection), residual_scale (float, default 1), tile_min_len (as ``PagedAttention``), rot_dim
-    (int, default 0: the turned part of a query head and the shared turned key part), rot_base (float),
-    rot_scaling (None or a rule of ``rotary_frequencies``), window (int, default 0: all keys)."""
+    (int, default 0: the turned part of a query head and the shared turned key part), rot_dims (int, default
+    rot_dim: how many of its coordinates turn, the first ones), rot_base (float), rot_scaling (None or a rule of ``rotary_frequencies``), window (int, default 0: all keys)."""
 
     raw_output_ok = True     # forward(..., residual32=None) returns the mixer's result alone
 
@@ -66,9 +66,13 @@ class LatentAttention(PagedAttention):
             raise ValueError("a latent attention with a turned key part caches it with its own latent")
         self._freq_host = self.freq = None
         if self.rot_dim:
-            freq, mult = rotary_frequencies(self.rot_dim, float(p["rot_base"]), p.get("rot_scaling"))
+            dims = int(p.get("rot_dims", self.rot_dim) or self.rot_dim)
+            if dims % 2 or not 0 < dims <= self.rot_dim:
+                raise ValueError(f"{dims} turning coordinates in a part of {self.rot_dim}")
+            freq, mult = rotary_frequencies(dims, float(p["rot_base"]), p.get("rot_scaling"))
             if mult != 1.0:
                 raise ValueError("this rule of rescaled frequencies also scales cosine and sine; not offered here")
+            freq = list(freq) + [0.0] * ((self.rot_dim - dims) // 2)      # an angle of zero leaves a pair as it is
             self._freq_host = torch.tensor(freq, dtype=torch.float64).to(torch.float32)
 
     def tensor_specs(self) -> List[TensorSpec]:

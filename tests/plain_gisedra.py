@@ -11,12 +11,47 @@ Notation: T tokens of one sequence, positions 0 .. T-1; h [T, width] is what a s
 """
 from __future__ import annotations
 
+import json
 import math
+import os
+import struct
 from typing import Dict, List, Optional
 
+import numpy as np
 import torch
 
 F64 = torch.float64
+
+
+# ----------------------------------------------------------------------------- files
+def read_safetensors(path: str) -> Dict[str, torch.Tensor]:
+    """8-byte little-endian header length, JSON header, raw data: name -> float64 (or int64) tensor."""
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(n))
+        blob = f.read()
+    out = {}
+    for name, info in header.items():
+        if name == "__metadata__":
+            continue
+        lo, hi = info["data_offsets"]
+        raw = np.frombuffer(blob[lo:hi], dtype=np.uint8)
+        if info["dtype"] == "BF16":
+            t = torch.from_numpy((raw.view("<u2").astype(np.uint32) << 16).view(np.float32).astype(np.float64))
+        elif info["dtype"] == "F32":
+            t = torch.from_numpy(raw.view("<f4").astype(np.float64))
+        elif info["dtype"] == "I32":
+            t = torch.from_numpy(raw.view("<i4").astype(np.int64))
+        else:
+            raise ValueError(f"{name}: dtype {info['dtype']}")
+        out[name] = t.reshape(info["shape"])
+    return out
+
+
+def load_folder(folder: str):
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    return cfg, read_safetensors(os.path.join(folder, "model.safetensors"))
 
 
 # ----------------------------------------------------------------------------- small functions
@@ -163,7 +198,7 @@ def latent_attention(h, W: Dict[str, torch.Tensor], p: str, c: dict, eps: float)
     q = (h @ W[p + ".q"].T).view(T, H, d + r)
     down = h @ W[p + ".dkv"].T
     lat = unit_rms(down[:, :R], eps) * W[p + ".dkv.norm"]
-    f = rotary_frequencies(r, c["rot"]["base"], c["rot"].get("scaling"))
+    f = rotary_frequencies(c["rot"]["dims"], c["rot"]["base"], c["rot"].get("scaling"))
     pos = torch.arange(T)
     k_rot = rotate(down[:, R:].view(T, 1, r), pos, f, True)
     q_rot = rotate(q[..., d:], pos, f, True)
@@ -249,3 +284,23 @@ def forward(tokens, weights: Dict[str, torch.Tensor], cfg: dict, streams: Option
         if streams is not None:
             streams.append(x.clone())
     return _norm(x, W, "final.norm") @ W["head"].T
+
+
+def logits(cfg: dict, w: Dict[str, torch.Tensor], tokens) -> torch.Tensor:
+    return forward(tokens, w, cfg)
+
+
+def residual_streams(cfg: dict, w: Dict[str, torch.Tensor], tokens) -> List[torch.Tensor]:
+    out: List[torch.Tensor] = []
+    forward(tokens, w, cfg, out)
+    return out
+
+
+def generate(cfg: dict, w: Dict[str, torch.Tensor], prompt, n: int) -> List[int]:
+    """Greedy continuation of ``prompt`` by ``n`` tokens (the lowest id on ties)."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(torch.argmax(logits(cfg, w, seq)[-1]))
+        out.append(nxt)
+        seq.append(nxt)
+    return out
