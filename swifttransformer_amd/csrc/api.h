@@ -224,8 +224,10 @@ int st_moe_combine(float* out, const float* residual, const float* pair_out, con
 // ---- float operations on the residual stream (csrc/stream_ops.hip)
 // y = tanh(alpha[0] * x[row]) * w + b (b may be null) of every row, or of the rows picked by `rows`
 // (negative: skipped); base != null: y += base[row of the result]; out32 (float) and / or out_t (`dtype`).
+// w2 != null: out_t receives tanh(alpha2[0] * y) * w2 + b2 instead of y (out32 still y).
 int st_dynamic_tanh(void* out_t, float* out32, const float* x, const int* rows, const float* w, const float* b,
-                    const float* alpha, const float* base, int num_rows, int width, int dtype, hipStream_t stream);
+                    const float* alpha, const float* base, const float* w2, const float* b2, const float* alpha2,
+                    int num_rows, int width, int dtype, hipStream_t stream);
 // x[t] += y[t] * rsqrt(mean(y[t]^2) + eps) * w
 int st_unit_add(float* x, const float* y, const float* w, int num_rows, int width, float eps, hipStream_t stream);
 // out[t] = x[t] (+ first[t]) + vec

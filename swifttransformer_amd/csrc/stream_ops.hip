@@ -2,7 +2,9 @@
 //
 //   dynamic tanh   y = tanh(alpha x) * w + b   per element (no mean, no variance), alpha one number on
 //                  the device; optionally of picked rows, optionally added to a second stream
-//                  (out32 = base + y: a branch's result normalised on its way into the stream);
+//                  (out32 = base + y: a branch's result normalised on its way into the stream), and
+//                  optionally followed by a second dynamic tanh of that sum in the storage type (what
+//                  the next sublayer reads), so that norm-after, residual sum and norm-before are one pass;
 //   unit add       x += y / sqrt(mean(y^2) + eps) * w   per row (a branch that enters the stream at
 //                  unit root mean square);
 //   row add        out = x (+ first) + vec   (a pass over a group of layers that starts from the stream
@@ -18,7 +20,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void dynamic_tanh_kernel(
     T* __restrict__ out_t, float* __restrict__ out32, const float* __restrict__ x, const int* __restrict__ rows,
     const float* __restrict__ w, const float* __restrict__ b, const float* __restrict__ alpha,
-    const float* __restrict__ base, int width, int64_t total) {
+    const float* __restrict__ base, const float* __restrict__ w2, const float* __restrict__ b2,
+    const float* __restrict__ alpha2, int width, int64_t total) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     const int64_t r = idx / width;
@@ -31,6 +34,7 @@ __global__ __launch_bounds__(256) void dynamic_tanh_kernel(
     float y = tanhf(alpha[0] * x[src * width + c]) * w[c] + (b ? b[c] : 0.f);
     if (base) y += base[idx];
     if (out32) out32[idx] = y;
+    if (w2) y = tanhf(alpha2[0] * y) * w2[c] + (b2 ? b2[c] : 0.f);     // the next norm, of the sum just made
     if (out_t) Elem<T>::store(out_t + idx, y);
 }
 
@@ -63,17 +67,19 @@ __global__ __launch_bounds__(256) void row_add_kernel(float* __restrict__ out, c
 using namespace st;
 
 extern "C" int st_dynamic_tanh(void* out_t, float* out32, const float* x, const int* rows, const float* w,
-                               const float* b, const float* alpha, const float* base, int num_rows, int width,
-                               int dtype, hipStream_t stream) {
+                               const float* b, const float* alpha, const float* base, const float* w2,
+                               const float* b2, const float* alpha2, int num_rows, int width, int dtype,
+                               hipStream_t stream) {
     ST_CHECK(num_rows >= 0 && width > 0, "dynamic_tanh: bad sizes");
     if (num_rows == 0) return 0;
     ST_CHECK(x && w && alpha && (out_t || out32), "dynamic_tanh: null operand");
+    ST_CHECK(!w2 || (alpha2 && out_t), "dynamic_tanh: a second norm needs its alpha and the storage-type output");
     const int64_t total = (int64_t)num_rows * width;
     const unsigned grid = (unsigned)((total + 255) / 256);
     if (dtype == kF32)
-        dynamic_tanh_kernel<float><<<grid, 256, 0, stream>>>((float*)out_t, out32, x, rows, w, b, alpha, base, width, total);
+        dynamic_tanh_kernel<float><<<grid, 256, 0, stream>>>((float*)out_t, out32, x, rows, w, b, alpha, base, w2, b2, alpha2, width, total);
     else if (dtype == kBF16)
-        dynamic_tanh_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out_t, out32, x, rows, w, b, alpha, base, width, total);
+        dynamic_tanh_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out_t, out32, x, rows, w, b, alpha, base, w2, b2, alpha2, width, total);
     else ST_CHECK(false, "dynamic_tanh: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("dynamic_tanh");
     return 0;

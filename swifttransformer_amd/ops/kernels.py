@@ -99,7 +99,8 @@ def _lib():
         lib.st_moe_down.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                     _c_f, _c_int, _c_p]
         lib.st_moe_combine.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_f, _c_p]
-        lib.st_dynamic_tanh.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_dynamic_tanh.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int,
+                                        _c_int, _c_p]
         lib.st_unit_add.argtypes = [_c_p, _c_p, _c_p, _c_int, _c_int, _c_f, _c_p]
         lib.st_row_add.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_p]
         if torch.cuda.is_available():
@@ -799,8 +800,9 @@ def token_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx_a
 
 
 # ------------------------------------------- rotary positions, one-pool page write
-@_timed("rotary", lambda q, k, *a, **kw: {"rows": q.shape[0], "width": q.shape[1] + k.shape[1],
-                                          "bytes": 2 * q.shape[0] * (q.shape[1] + k.shape[1]) * q.element_size()})
+@_timed("rotary", lambda q, k, *a, **kw: {"rows": q.shape[0], "width": q.shape[1] + (k.shape[1] if k is not None else 0),
+                                          "bytes": 2 * q.shape[0] * (q.shape[1] + (k.shape[1] if k is not None else 0)) *
+                                                   q.element_size()})
 def rotary(q: torch.Tensor, k: Optional[torch.Tensor], head_dim: int, freq: torch.Tensor, mult: float,
            positions: torch.Tensor, offset: int = 0, interleaved: bool = False) -> None:
     """In place on q [T, heads * head_dim] and k [T, kv_heads * head_dim] (dense rows, any row stride; k may
@@ -1243,10 +1245,13 @@ def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, 
                                             (k.get("rows").shape[0] if k.get("rows") is not None else x.shape[0])})
 def dynamic_tanh(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], alpha: torch.Tensor, *,
                  rows: Optional[torch.Tensor] = None, out_t: Optional[torch.Tensor] = None,
-                 out_f32: Optional[torch.Tensor] = None, base: Optional[torch.Tensor] = None) -> None:
+                 out_f32: Optional[torch.Tensor] = None, base: Optional[torch.Tensor] = None,
+                 then: Optional[tuple] = None) -> None:
     """y = tanh(alpha * x) * weight + bias per element of the float rows x [T, width] (of the rows picked by
     ``rows``, int32, negative entries skipped); ``alpha``: float [1] on the device.  ``base`` (float, the
-    result's shape): y += base.  Written to ``out_f32`` (float) and / or ``out_t`` (float or bfloat16)."""
+    result's shape): y += base.  Written to ``out_f32`` (float) and / or ``out_t`` (float or bfloat16).
+    ``then`` = (weight2, bias2 or None, alpha2): ``out_t`` receives tanh(alpha2 * y) * weight2 + bias2
+    instead of y (``out_f32`` still y)."""
     T, W = x.shape
     n = rows.shape[0] if rows is not None else T
     _need(x, "x", torch.float32, (T, W))
@@ -1264,8 +1269,18 @@ def dynamic_tanh(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
         _need(out_t, "out_t", None, (n, W))
     if base is not None:
         _need(base, "base", torch.float32, (n, W))
+    w2 = b2 = a2 = None
+    if then is not None:
+        w2, b2, a2 = then
+        _need(w2, "weight2", torch.float32, (W,))
+        if b2 is not None:
+            _need(b2, "bias2", torch.float32, (W,))
+        _need(a2, "alpha2", torch.float32, (1,))
+        if out_t is None:
+            raise KernelError("dynamic_tanh: the second norm goes to out_t")
     _check(_lib().st_dynamic_tanh(_ptr(out_t), _ptr(out_f32), _ptr(x), _ptr(rows), _ptr(weight), _ptr(bias), _ptr(alpha),
-                                  _ptr(base), n, W, dtype_code(out_t.dtype) if out_t is not None else F32, _stream()))
+                                  _ptr(base), _ptr(w2), _ptr(b2), _ptr(a2), n, W,
+                                  dtype_code(out_t.dtype) if out_t is not None else F32, _stream()))
 
 
 @_timed("unit_add", lambda x, y, *a, **k: {"rows": x.shape[0], "width": x.shape[1], "bytes": 12 * x.numel()})

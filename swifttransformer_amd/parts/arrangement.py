@@ -83,11 +83,30 @@ class Sandwich(Part):
                 raise ValueError(f"{type(part).__name__} cannot give its result without the residual stream")
         a, _ = layer.mixer_norm.forward(x32, out_t=True)
         m32 = layer.mixer.forward(a, None, ctx, cache, write)
-        x32 = layer.mixer_out_norm.forward_onto(m32, x32)
+        side = layer.side_input
+        x_t = None                                  # the stream in the storage type, where a pass has made it
         if self.has_ffn:
-            d, _ = layer.ffn_norm.forward(x32, out_t=True)
+            # norm after the mixer, the sum into the stream and the norm before the feed-forward: one pass where
+            # the two norms can do that
+            if _chains(layer.mixer_out_norm, layer.ffn_norm):
+                x32, d = layer.mixer_out_norm.forward_onto(m32, x32, then=layer.ffn_norm)
+            else:
+                x32 = layer.mixer_out_norm.forward_onto(m32, x32)
+                d, _ = layer.ffn_norm.forward(x32, out_t=True)
             f32 = layer.feed_forward.forward(d, None, ctx)
-            x32 = layer.ffn_out_norm.forward_onto(f32, x32)
-        if layer.side_input is not None:
-            x32 = layer.side_input.forward(x32, ctx)
+            last = layer.ffn_out_norm
+        else:
+            f32, last = m32, layer.mixer_out_norm
+        if side is not None and _chains(last, None):
+            x32, x_t = last.forward_onto(f32, x32, cast=True)
+        else:
+            x32 = last.forward_onto(f32, x32)
+        if side is not None:
+            x32 = side.forward(x32, ctx, x_t=x_t)
         return x32
+
+
+def _chains(norm, then) -> bool:
+    """Whether ``norm.forward_onto`` can make a second result in the same pass (``then``: another norm of its
+    kind, or None for the plain sum in the storage type)."""
+    return getattr(norm, "chains_onto", False) and (then is None or type(then) is type(norm))

@@ -32,7 +32,7 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
                 that has a ``mixer_conv`` part)
   token_conv    ``cache_need() -> CacheNeed``; ``forward(y32, ctx, cache) -> y_t``: a short causal
                 filter over time on what a mixer reads, with its last inputs as per-request state
-  side_input    ``forward(x32, ctx) -> x32``: what a layer adds to the stream after its feed-forward
+  side_input    ``forward(x32, ctx, x_t=None) -> x32`` (``x_t``: the stream in the storage type, if at hand): what a layer adds to the stream after its feed-forward
                 from an input of the token's own (a per-layer token embedding)
   reentry       ``forward(x32, first32, ctx) -> x32``: what happens to the residual stream before a run
                 of a layer that the schedule marks (``ScheduleEntry.enter``); ``first32`` is the

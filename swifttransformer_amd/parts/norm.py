@@ -80,6 +80,8 @@ class DynamicTanh(Part):
     """params: width (int, default hidden_size), bias (bool, default True).  names: weight, bias, alpha
     (a tensor of no dimensions)."""
 
+    chains_onto = True      # forward_onto(..., then=another of this kind / cast=True) makes a second result in its pass
+
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
         self.width = int(self.param("width", hidden_size))
@@ -111,8 +113,18 @@ class DynamicTanh(Part):
         K.dynamic_tanh(x32, self.gamma, self.beta, self.alpha, rows=rows, out_t=yt, out_f32=y32)
         return (y32, y32) if both else (yt, y32)
 
-    def forward_onto(self, y32: torch.Tensor, stream32: torch.Tensor) -> torch.Tensor:
-        """stream32 + norm(y32), float, a new tensor."""
+    def forward_onto(self, y32: torch.Tensor, stream32: torch.Tensor, then=None, cast: bool = False):
+        """stream32 + norm(y32), float, a new tensor.  ``then`` (another ``DynamicTanh``): returns (the sum, that
+        norm of the sum in the storage type), made in the same pass; ``cast``: (the sum, the sum in the storage
+        type)."""
         out = K.empty(tuple(stream32.shape), torch.float32, stream32.device)
-        K.dynamic_tanh(y32, self.gamma, self.beta, self.alpha, out_f32=out, base=stream32)
-        return out
+        if then is None and not cast:
+            K.dynamic_tanh(y32, self.gamma, self.beta, self.alpha, out_f32=out, base=stream32)
+            return out
+        if self.dtype == torch.float32 and then is None:
+            K.dynamic_tanh(y32, self.gamma, self.beta, self.alpha, out_f32=out, base=stream32)
+            return out, out
+        out_t = K.empty(tuple(stream32.shape), self.dtype, stream32.device)
+        K.dynamic_tanh(y32, self.gamma, self.beta, self.alpha, out_f32=out, out_t=out_t, base=stream32,
+                       then=None if then is None else (then.gamma, then.beta, then.alpha))
+        return out, out_t

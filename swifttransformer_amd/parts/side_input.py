@@ -43,9 +43,11 @@ class TokenSideInput(Part):
         self.table = tensors[self.name("table")][:, lo:lo + self.dim].contiguous()    # this layer's columns
         self.w_gate, self.w_proj, self.gain = (tensors[self.name(n)] for n in ("gate", "proj", "norm"))
 
-    def forward(self, x32: torch.Tensor, ctx) -> torch.Tensor:
+    def forward(self, x32: torch.Tensor, ctx, x_t: torch.Tensor = None) -> torch.Tensor:
+        """``x_t``: the stream in the storage type, where the caller has it already."""
         T = x32.shape[0]
-        x_t = x32 if self.dtype == torch.float32 else K.cast(x32, self.dtype)
+        if x_t is None:
+            x_t = x32 if self.dtype == torch.float32 else K.cast(x32, self.dtype)
         e = K.empty((T, self.dim), self.dtype, x32.device)
         K.lookup(ctx.token_ids, self.table, out_f32=e if self.dtype == torch.float32 else None,
                  out_t=None if self.dtype == torch.float32 else e)
