@@ -86,6 +86,8 @@ class ModelRunner:
         if max_batched_tokens is None:
             max_batched_tokens = min(model.max_positions, 2048) + max(0, cache_param.max_seqs - 1)
         self.max_batched_tokens = int(max_batched_tokens)
+        # a recorded step has the rows of its batch's bucket: the arena holds such a step too
+        self.arena_rows = token_bucket(max(1, self.max_batched_tokens))
         self.arena = StepArena(self.device)
         if self.device.type == "cuda" and model.weights_loaded:
             self._size_arena(cache_param)
@@ -115,7 +117,7 @@ class ModelRunner:
         """Measure what a step of ``max_batched_tokens`` tokens makes per layer (one run through the
         ordinary allocator on a one-page cache of its own: a prompt portion as long as the model
         allows, the rest single tokens), and allocate the arena's two banks for it."""
-        T = max(1, self.max_batched_tokens)
+        T = max(1, self.arena_rows)
         ps = cache_param.page_size
         P = min(self.model.max_positions, self.max_pages_per_seq * ps)
         first = min(T, P)
@@ -309,14 +311,19 @@ class ModelRunner:
         with using_arena(self.arena):
             if tune:
                 with K.tuned_products():
-                    run()
+                    first = run()
             else:
-                run()
+                first = run()
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph), using_arena(self.arena):
             out = run()
             state = self.arena.state()
+        # A tensor that did not fit the arena came from the ordinary allocator in the first run and from
+        # the recording's own pool in the second: the first run's result is then not where the recording
+        # leaves it, and this batch's caller reads it there.
+        if out.data_ptr() != first.data_ptr():
+            out.copy_(first)
         return _RecordedStep(buffers, graph, out, state, best)
 
     # ----------------------------------------- recorded steps of any composition

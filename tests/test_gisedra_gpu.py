@@ -390,6 +390,30 @@ def test_peaked_latent_attention_at_window_edges_page_borders_and_far_back(model
     assert all(g.pool.num_free == g.pool.num_pages for g in runner.manager.paged_groups)
 
 
+def test_the_step_that_is_recorded_gives_its_own_result_also_where_its_tensors_left_the_arena(models, dtype="float32"):
+    """A step's bucket of rows may be larger than the most tokens the runner was built for, and a tensor that
+    does not fit the arena comes from the ordinary allocator: the batch whose step is recorded must read the
+    result of its own run, not the recording's untouched memory."""
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.batch import token_bucket
+    from swifttransformer_amd.engine.step import ModelRunner
+    from swifttransformer_amd.models import load_model
+    folder, cfg, w = models["A"]
+    seqs = {0: tiny.prompt(70, cfg["vocab"], 21), 1: tiny.prompt(66, cfg["vocab"], 22)}      # one bucket: 128 rows
+    refs = {r: plain.logits(cfg, w, s).numpy() for r, s in seqs.items()}
+    ps = tiny.PAGE_SIZE["A"]
+    model = load_model(folder, DTYPES[dtype], DEV)
+    runner = ModelRunner(model, CacheParam(page_size=ps, num_pages=40, max_seqs=4), DEV, record_after=2, max_batched_tokens=70)
+    assert runner.arena_rows == token_bucket(70) == 128
+    run_schedule(runner, seqs, refs, [[(0, 70)], [(1, 66)], [(0, 70)], [(1, 66)]], dtype, f"{dtype} in the arena")
+    assert runner.arena.overflows == 0 and runner.graph_replays == 3
+    # nothing fits: every tensor of the first run and of the recording comes from elsewhere
+    runner = ModelRunner(model, CacheParam(page_size=ps, num_pages=40, max_seqs=4), DEV, record_after=2, max_batched_tokens=70)
+    runner.arena.resize(256)
+    run_schedule(runner, seqs, refs, [[(0, 70)], [(1, 66)], [(0, 70)], [(1, 66)]], dtype, f"{dtype} outside the arena")
+    assert runner.arena.overflows > 0 and runner.graph_replays == 3
+
+
 def test_greedy_generation_through_the_engine(models):
     from swifttransformer_amd.engine.engine import Engine
     from swifttransformer_amd.sampling import SamplingParams
