@@ -234,6 +234,13 @@ int st_unit_add(float* x, const float* y, const float* w, int num_rows, int widt
 int st_row_add(float* out, const float* x, const float* first, const float* vec, int num_rows, int width,
                hipStream_t stream);
 
+// x[t] += unit(P (gelu_tanh(G x[t]) * table[token_ids[t], :dim])) * gain, unit(y) = y * rsqrt(mean(y^2) + eps).
+// table rows of `table_stride` elements, w_gate [dim, width], w_proj [width, dim] of `dtype`; x, gain float.
+// Rows with token_item[t] < 0 (if given) are left alone; a token outside the table gates with zeros.
+int st_token_side(float* x, const int* token_ids, const int* token_item, const void* table, int64_t table_stride,
+                  int vocab, const void* w_gate, const void* w_proj, const float* gain, int num_rows, int dim,
+                  int width, float eps, int dtype, hipStream_t stream);
+
 // Measurement kernels (csrc/probe.hip): a plain streaming read, and a kernel without work.
 int st_probe_read(const void* src, int64_t bytes, void* sink, int workgroups, int pattern, hipStream_t stream);
 int st_probe_empty(void* sink, hipStream_t stream);

@@ -9,8 +9,13 @@
 //                  unit root mean square);
 //   row add        out = x (+ first) + vec   (a pass over a group of layers that starts from the stream
 //                  plus the step's embedding plus that pass's vector).
+//   token side     x += unit(P (gelu_tanh(G x) * e[token])) * w   per row: a narrow embedding row gates a
+//                  projection of the stream, which re-enters it at unit root mean square; lookup, the two
+//                  small products, the activation, the norm and the sum in one kernel.
 //
-// Everything is float except the optional copy of the dynamic tanh in the storage type.
+// Everything is float except the optional copy of the dynamic tanh in the storage type and the token side
+// input's two products, whose operands are of the storage type (sums in float).
+#include "activation.h"
 #include "api.h"
 #include "common.h"
 
@@ -62,6 +67,77 @@ __global__ __launch_bounds__(256) void row_add_kernel(float* __restrict__ out, c
     out[idx] = v + vec[idx % width];
 }
 
+template <typename T> __device__ inline float as_stored(float v);
+template <> __device__ inline float as_stored<float>(float v) { return v; }
+template <> __device__ inline float as_stored<bf16_t>(float v) { return bf16_to_float(float_to_bf16(v)); }
+
+// A workgroup a row: 16 waves where rows are few (a decode step: every gate feature's row of G in flight
+// at once, the kernel's time a handful of dependent trips to memory), 4 otherwise.  LDS: the row in the
+// storage type's values (as floats), later the projection's result; the gated vector.
+// g_j = stored(gelu(stored(G_j . x)) * e_j), y = P g, x += y / sqrt(mean(y^2) + eps) * w.
+// VEC: rows of G and P allow 16-byte loads.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(1024) void token_side_kernel(
+    float* __restrict__ x, const int* __restrict__ token_ids, const int* __restrict__ token_item,
+    const T* __restrict__ table, int64_t table_stride, int vocab, const T* __restrict__ w_gate,
+    const T* __restrict__ w_proj, const float* __restrict__ gain, int dim, int width, float eps) {
+    extern __shared__ __attribute__((aligned(16))) float side_lds[];
+    __shared__ float red[16];
+    float* xs = side_lds;                 // [width]
+    float* gs = side_lds + width;         // [dim]
+    const int64_t row = blockIdx.x;
+    if (token_item && token_item[row] < 0) return;        // a padding row (uniform over the workgroup)
+    constexpr int V = Elem<T>::kVec;
+    const int threads = blockDim.x, waves = threads >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float* xr = x + row * width;
+    const int tok = token_ids[row];
+    const bool known = tok >= 0 && tok < vocab;
+    const T* er = table + (int64_t)(known ? tok : 0) * table_stride;
+    // the first feature's table entry is asked for before the row arrives
+    float e = (known && wave < dim) ? Elem<T>::load(er + wave) : 0.f;
+    for (int c = threadIdx.x; c < width; c += threads) xs[c] = as_stored<T>(xr[c]);
+    __syncthreads();
+    for (int j = wave; j < dim; j += waves) {
+        const T* gr = w_gate + (int64_t)j * width;
+        float acc = 0.f;
+        if (VEC) {
+            for (int c = lane * V; c < width; c += 64 * V) {
+                float w[V];
+                Elem<T>::load_vec(gr + c, w);
+#pragma unroll
+                for (int u = 0; u < V; ++u) acc = fmaf(w[u], xs[c + u], acc);
+            }
+        } else {
+            for (int c = lane; c < width; c += 64) acc = fmaf(Elem<T>::load(gr + c), xs[c], acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) gs[j] = as_stored<T>(apply_activation(kActGeluTanh, as_stored<T>(acc)) * e);
+        if (j + waves < dim) e = known ? Elem<T>::load(er + j + waves) : 0.f;
+    }
+    __syncthreads();                      // every wave has read xs; gs is complete
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += threads) {
+        const T* pr = w_proj + (int64_t)c * dim;
+        float y = 0.f;
+        if (VEC) {
+            for (int j = 0; j < dim; j += V) {
+                float w[V];
+                Elem<T>::load_vec(pr + j, w);
+#pragma unroll
+                for (int u = 0; u < V; ++u) y = fmaf(w[u], gs[j + u], y);
+            }
+        } else {
+            for (int j = 0; j < dim; ++j) y = fmaf(Elem<T>::load(pr + j), gs[j], y);
+        }
+        xs[c] = y;                        // this thread's own entries from here on
+        ss = fmaf(y, y, ss);
+    }
+    ss = block_sum(ss, red);
+    const float r = 1.f / sqrtf(ss / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += threads) xr[c] += xs[c] * r * gain[c];
+}
+
 }  // namespace st
 
 using namespace st;
@@ -103,5 +179,33 @@ extern "C" int st_row_add(float* out, const float* x, const float* first, const 
     const int64_t total = (int64_t)num_rows * width;
     row_add_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(out, x, first, vec, width, total);
     ST_LAUNCH_CHECK("row_add");
+    return 0;
+}
+
+extern "C" int st_token_side(float* x, const int* token_ids, const int* token_item, const void* table,
+                             int64_t table_stride, int vocab, const void* w_gate, const void* w_proj,
+                             const float* gain, int num_rows, int dim, int width, float eps, int dtype,
+                             hipStream_t stream) {
+    ST_CHECK(num_rows >= 0 && width > 0 && dim > 0 && vocab > 0 && eps > 0.f && table_stride >= dim,
+             "token_side: bad sizes");
+    ST_CHECK(dtype == kF32 || dtype == kBF16, "token_side: unknown dtype %d", dtype);
+    const size_t lds = sizeof(float) * ((size_t)width + dim);
+    ST_CHECK(lds <= 60 * 1024, "token_side: a row of %d and a gated vector of %d do not fit the LDS", width, dim);
+    if (num_rows == 0) return 0;
+    ST_CHECK(x && token_ids && table && w_gate && w_proj && gain, "token_side: null operand");
+    const int threads = num_rows <= 256 ? 1024 : 256;
+    const int vec = dtype == kF32 ? 4 : 8;
+    const bool aligned = width % vec == 0 && dim % vec == 0 && (uintptr_t)w_gate % 16 == 0 && (uintptr_t)w_proj % 16 == 0;
+#define ST_SIDE(T, VEC)                                                                                          \
+    token_side_kernel<T, VEC><<<(unsigned)num_rows, threads, lds, stream>>>(                                         \
+        x, token_ids, token_item, (const T*)table, table_stride, vocab, (const T*)w_gate, (const T*)w_proj, gain, dim, \
+        width, eps)
+    if (dtype == kF32) {
+        if (aligned) ST_SIDE(float, true); else ST_SIDE(float, false);
+    } else {
+        if (aligned) ST_SIDE(bf16_t, true); else ST_SIDE(bf16_t, false);
+    }
+#undef ST_SIDE
+    ST_LAUNCH_CHECK("token_side");
     return 0;
 }

@@ -102,6 +102,8 @@ def _lib():
         lib.st_dynamic_tanh.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int,
                                         _c_int, _c_p]
         lib.st_unit_add.argtypes = [_c_p, _c_p, _c_p, _c_int, _c_int, _c_f, _c_p]
+        lib.st_token_side.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
+                                      _c_f, _c_int, _c_p]
         lib.st_row_add.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
@@ -1291,6 +1293,40 @@ def unit_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float)
     _need(y, "y", torch.float32, (T, W))
     _need(weight, "weight", torch.float32, (W,))
     _check(_lib().st_unit_add(_ptr(x), _ptr(y), _ptr(weight), T, W, float(eps), _stream()))
+    return x
+
+
+def token_side_fits(width: int, dim: int) -> bool:
+    """Whether ``token_side`` takes these sizes: a row and the gated vector as floats in 60 KB of LDS."""
+    return 4 * (width + dim) <= 60 * 1024
+
+
+@_timed("token_side", lambda x, ids, item, table, w_gate, *a, **k: {
+    "rows": x.shape[0], "width": x.shape[1], "inner": w_gate.shape[0],
+    "bytes": 8 * x.numel() + 2 * w_gate.numel() * w_gate.element_size()})
+def token_side(x: torch.Tensor, token_ids: torch.Tensor, token_item: Optional[torch.Tensor], table: torch.Tensor,
+               w_gate: torch.Tensor, w_proj: torch.Tensor, gain: torch.Tensor, eps: float) -> torch.Tensor:
+    """x[t] += unit(w_proj (gelu_tanh(w_gate x[t]) * table[token_ids[t]])) * gain, in place on the float rows x
+    [T, width]; unit(y) = y / sqrt(mean(y^2) + eps).  table [vocab, dim] (rows may be strided: columns of a wider
+    table), w_gate [dim, width], w_proj [width, dim] of one storage type: the two products take operands of that
+    type (x rounded to it) and sum in float.  Rows with token_item < 0 are left alone."""
+    T, W = x.shape
+    dim = w_gate.shape[0]
+    _need(x, "x", torch.float32, (T, W))
+    _need(token_ids, "token_ids", torch.int32, (T,))
+    if token_item is not None:
+        _need(token_item, "token_item", torch.int32, (T,))
+    dt = w_gate.dtype
+    _need(w_gate, "w_gate", dt, (dim, W))
+    _need(w_proj, "w_proj", dt, (W, dim))
+    _need(table, "table", dt, (table.shape[0], dim), contiguous=False)
+    if table.stride(1) != 1:
+        raise KernelError("table: rows must be dense")
+    _need(gain, "gain", torch.float32, (W,))
+    if not token_side_fits(W, dim):
+        raise KernelError(f"token_side: a row of {W} and a gated vector of {dim} do not fit the LDS")
+    _check(_lib().st_token_side(_ptr(x), _ptr(token_ids), _ptr(token_item), _ptr(table), table.stride(0), table.shape[0],
+                                _ptr(w_gate), _ptr(w_proj), _ptr(gain), T, dim, W, float(eps), dtype_code(dt), _stream()))
     return x
 
 

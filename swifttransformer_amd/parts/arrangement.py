@@ -97,7 +97,7 @@ class Sandwich(Part):
             last = layer.ffn_out_norm
         else:
             f32, last = m32, layer.mixer_out_norm
-        if side is not None and _chains(last, None):
+        if side is not None and not getattr(side, "fused", False) and _chains(last, None):
             x32, x_t = last.forward_onto(f32, x32, cast=True)
         else:
             x32 = last.forward_onto(f32, x32)

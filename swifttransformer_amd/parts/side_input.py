@@ -4,8 +4,10 @@ stream and re-enters it at unit root mean square.
     e = E[token, index * dim : (index + 1) * dim]         one table for all layers, a part of a row a layer
     g = gelu_tanh(G x) * e;  y = P g;  x <- x + y / rms(y) * s
 
-The two products take the engine's storage type; the unit norm and the sum into the stream are float.
-The reference has no such part."""
+The two products take the engine's storage type (sums in float); the unit norm and the sum into the stream
+are float.  One kernel a row does all of it (``token_side``: the row in LDS, a wave a gate feature, a thread
+an output feature); a stream wider than that kernel's LDS takes the separate kernels.  The reference has
+no such part."""
 from __future__ import annotations
 
 from typing import Dict, List
@@ -40,11 +42,17 @@ class TokenSideInput(Part):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         lo = self.index * self.dim
-        self.table = tensors[self.name("table")][:, lo:lo + self.dim].contiguous()    # this layer's columns
+        self.table = tensors[self.name("table")][:, lo:lo + self.dim]     # this layer's columns of the shared table
+        self.fused = K.token_side_fits(self.hidden_size, self.dim)
+        if not self.fused:
+            self.table = self.table.contiguous()
         self.w_gate, self.w_proj, self.gain = (tensors[self.name(n)] for n in ("gate", "proj", "norm"))
 
     def forward(self, x32: torch.Tensor, ctx, x_t: torch.Tensor = None) -> torch.Tensor:
         """``x_t``: the stream in the storage type, where the caller has it already."""
+        if self.fused:
+            return K.token_side(x32, ctx.token_ids, ctx.token_item, self.table, self.w_gate, self.w_proj, self.gain,
+                                self.eps)
         T = x32.shape[0]
         if x_t is None:
             x_t = x32 if self.dtype == torch.float32 else K.cast(x32, self.dtype)

@@ -90,6 +90,35 @@ def test_rotary_interleaved_from_an_offset_and_latent_write_with_a_turned_tail(d
     check(cache[3, 0, 1][None, rank:rank + tail], x[1, rank:][None].to(F64).numpy(), dt, "plain tail")
 
 
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("W,dim,parts,index", [(64, 8, 3, 1), (72, 6, 2, 1), (100, 2, 1, 0), (2048, 16, 4, 3), (328, 20, 2, 0)])
+def test_token_side_input_in_one_kernel(dtype, W, dim, parts, index):
+    """Lookup, gate product, GELU, projection, unit norm and the sum into the stream: against the plain function, on
+    columns of a wider table, with a padding row, a token outside the table and sizes that no vector load divides."""
+    from swifttransformer_amd.ops import kernels as K
+    g = torch.Generator().manual_seed(W + dim)
+    dt = DTYPES[dtype]
+    T, V, eps = 11, 37, 1e-5
+    x = torch.randn(T, W, generator=g) * 1.5
+    tokens = torch.randint(0, V, (T,), generator=g)
+    weights = {"side.embed": rounded(torch.randn(V, parts * dim, generator=g), dtype),
+               f"l{index}.side.gate": rounded(torch.randn(dim, W, generator=g) / W ** 0.5, dtype),
+               f"l{index}.side.proj": rounded(torch.randn(W, dim, generator=g) / dim ** 0.5, dtype),
+               f"l{index}.side.norm": 0.5 + 0.1 * torch.randn(W, generator=g).to(F64)}
+    xs = rounded(x, dtype)                      # the products read the stream in the storage type
+    ref = x.to(F64) + plain.side_input(xs, tokens, weights, index, dim, eps)
+    ref[4] = x[4].to(F64)                       # a padding row stays as it is
+    item = torch.zeros(T, dtype=torch.int32)
+    item[4] = -1
+    ids = tokens.to(torch.int32)
+    ids[9] = V + 3                              # outside the table: gated with zeros, so y = 0 and x stays
+    ref[9] = x[9].to(F64)
+    table = dev(weights["side.embed"], dt)[:, index * dim:(index + 1) * dim]
+    got = K.token_side(dev(x).clone(), ids.to(DEV), item.to(DEV), table, dev(weights[f"l{index}.side.gate"], dt),
+                       dev(weights[f"l{index}.side.proj"], dt), dev(weights[f"l{index}.side.norm"]), eps)
+    check(got, ref.numpy(), dt, f"token side input, width {W}, {dim} of {parts * dim} columns", loosen=2.0)
+
+
 def plain_kept_window(q, k, v, scale, window, keep_first):
     T = q.shape[0]
     return plain.softmax_attention(q, k, v, scale, plain.visible(T, window, keep_first))
