@@ -159,6 +159,17 @@ int st_gated_group_norm(void* out, const float* o, const void* gate, int64_t gat
                         int num_tokens, int groups, int width, int gain_per_group, int gate_first, float eps,
                         int dtype, hipStream_t stream);
 
+// ---- retention in chunks (csrc/retention.hip): S <- decay_h S + (key_factor k) v^T, o = S^T q over each item's rows,
+// from and back to the item's state slot, as products within chunks of st_retention_chunk_rows(key_dim) rows and a
+// carry between them.  q, k float rows [heads * key_dim], v [heads * value_dim]; decay float [heads]; scratch: float
+// [scratch_chunks, heads, key_dim, value_dim] with scratch_chunks >= num_rows / chunk rows + num_items.
+int st_retention_chunk_rows(int key_dim);
+int st_retention_chunks(float* out, const float* q, int64_t q_stride, const float* k, int64_t k_stride, const float* v,
+                        int64_t v_stride, const float* decay, float key_factor, float* state, int64_t slot_stride,
+                        const int* item_len, const int* item_tok_off, const int* item_slot, int num_items, int num_rows,
+                        int heads, int key_dim, int value_dim, float* scratch, int64_t scratch_chunks,
+                        hipStream_t stream);
+
 // ---- gated linear attention (csrc/recurrent.hip)
 // out = sigmoid(z)^(inv_tau) over n floats (out may be z).
 int st_decay_gate(float* out, const float* z, int64_t n, float inv_tau, hipStream_t stream);

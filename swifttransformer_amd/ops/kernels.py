@@ -102,6 +102,9 @@ def _lib():
         lib.st_dynamic_tanh.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int,
                                         _c_int, _c_p]
         lib.st_unit_add.argtypes = [_c_p, _c_p, _c_p, _c_int, _c_int, _c_f, _c_p]
+        lib.st_retention_chunk_rows.argtypes = [_c_int]
+        lib.st_retention_chunks.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_f, _c_p, _c_i64,
+                                            _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p, _c_i64, _c_p]
         lib.st_token_side.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
                                       _c_f, _c_int, _c_p]
         lib.st_row_add.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_p]
@@ -1006,6 +1009,45 @@ def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate_a: torch.
                                 _ptr(gate_a), _ptr(gate_b), gate_stride, _ptr(skip), _ptr(state), slot_stride, _ptr(item_len),
                                 _ptr(item_tok_off), _ptr(item_slot), B, int(max_item_rows) or T, heads, qk_heads, kd, vd,
                                 {"additive": 0, "delta": 1}[mode], _stream()))
+    return out
+
+
+@_timed("retention_chunks", lambda q, k, v, decay, key_factor, state, ctx_arrays, heads: {
+    "rows": q.shape[0], "heads": heads, "key_dim": state.shape[2], "value_dim": state.shape[3],
+    "items": ctx_arrays[3].shape[0],
+    "bytes": 4 * (q.shape[0] * (q.shape[1] + k.shape[1] + 2 * v.shape[1]) +
+                  3 * (q.shape[0] // 16 + 1) * heads * state.shape[2] * state.shape[3])})
+def retention_chunks(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, key_factor: float,
+                     state: torch.Tensor, ctx_arrays, heads: int) -> torch.Tensor:
+    """Per item and head, from the slot's state S [key_dim, value_dim] and over the item's rows in order:
+    S <- decay[head] S + (key_factor k_t) v_t^T, o_t = S^T q_t; the state is stored back.  What ``state_scan``
+    computes in its additive form with constant gates, as products within chunks of rows and a carry between
+    chunks: for steps with prompts or portions.  q, k: float [T, heads * key_dim], v: float [T, heads * value_dim]
+    (dense rows, any stride); decay: float [heads]; state: float [slots, heads, key_dim, value_dim].  Returns
+    float [T, heads * value_dim]; rows of no item are left as they are."""
+    _token_item, item_len, item_tok_off, item_slot = ctx_arrays
+    T = q.shape[0]
+    _, sh, kd, vd = state.shape
+    if sh != heads or q.shape[1] != heads * kd or k.shape[1] != heads * kd or v.shape[1] != heads * vd:
+        raise KernelError("retention_chunks: the operands' sizes do not fit the state")
+    if kd > 256:
+        raise KernelError(f"retention_chunks: up to 256 key channels a head, not {kd}")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _need(t, name, torch.float32, (T, t.shape[1]), contiguous=False)
+        if t.stride(1) != 1:
+            raise KernelError(f"{name}: rows must be dense")
+    _need(decay, "decay", torch.float32, (heads,))
+    slot_stride = _slot_rows(state, "state", heads * kd * vd)
+    B = item_slot.shape[0]
+    for name, t in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
+        _need(t, name, torch.int32, (B,))
+    out = empty((T, heads * vd), torch.float32, q.device)
+    chunks = T // int(_lib().st_retention_chunk_rows(kd)) + B
+    scratch = empty((max(chunks, 1), heads, kd, vd), torch.float32, q.device)
+    _check(_lib().st_retention_chunks(_ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
+                                      _ptr(decay), float(key_factor), _ptr(state), slot_stride, _ptr(item_len),
+                                      _ptr(item_tok_off), _ptr(item_slot), B, T, heads, kd, vd, _ptr(scratch), chunks,
+                                      _stream()))
     return out
 
 

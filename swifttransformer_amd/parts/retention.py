@@ -4,9 +4,11 @@
     S_t = decay_h S_(t-1) + k_t v_t^T;  o_t = S_t^T q_t      (S float, one per request and head)
     y = Wo (concat_h(o_h / rms(o_h)) * silu(Wg x))
 
-The state lives in the request's state slot and is carried from step to step, so prompts, portions and
-decoded tokens run through the same kernel (``state_scan`` in its additive form, its two gates one row
-of constants: key_dim^-1/2 and the head's decay).  q, k and v leave their product as floats; the state,
+The state lives in the request's state slot and is carried from step to step.  Steps of single tokens and
+small steps run ``state_scan`` in its additive form (its two gates one row of constants: key_dim^-1/2 and
+the head's decay); steps of ``chunked_from`` rows or more that hold prompts or portions run
+``retention_chunks``: because the decay does not change over time, a chunk's own sums need no state and the
+chunks run side by side, with a carry of the state between them.  q, k and v leave their product as floats; the state,
 the sums over it and the heads' unit norm are float.  The reference has no such mixer."""
 from __future__ import annotations
 
@@ -24,6 +26,7 @@ class Retention(Mixer):
     unit norm), out_scale (float, default 1: a factor on the result)."""
 
     raw_output_ok = True
+    chunked_from = 64          # rows of a step from which prompts and portions take the chunked kernels
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
@@ -56,6 +59,7 @@ class Retention(Mixer):
         dev = self.w_out.device
         self.key_factor = torch.full((1, self.num_heads), float(self.key_dim) ** -0.5, dtype=torch.float32, device=dev)
         self.decays = torch.tensor([self.decay], dtype=torch.float64).to(torch.float32).to(dev)
+        self.decay_row = self.decays[0].contiguous()
         self.gain = torch.ones(self.value_dim, dtype=torch.float32, device=dev)
 
     def cache_need(self) -> CacheNeed:
@@ -69,7 +73,11 @@ class Retention(Mixer):
         items = (ctx.token_item, ctx.item_len, ctx.item_tok_off, ctx.item_slot)
         qkv = K.gemm(x_t, self.w_qkv, out_f32=True)
         gate = K.gemm(x_t, self.w_gate)
-        o = K.state_scan(qkv[:, :qk], qkv[:, qk:2 * qk], qkv[:, 2 * qk:], self.key_factor, self.decays, cache.state,
-                         items, self.num_heads, "additive", max_item_rows=1 if ctx.all_single else 0)
+        if not ctx.all_single and x_t.shape[0] >= self.chunked_from:
+            o = K.retention_chunks(qkv[:, :qk], qkv[:, qk:2 * qk], qkv[:, 2 * qk:], self.decay_row,
+                                   float(self.key_dim) ** -0.5, cache.state, items, self.num_heads)
+        else:
+            o = K.state_scan(qkv[:, :qk], qkv[:, qk:2 * qk], qkv[:, 2 * qk:], self.key_factor, self.decays, cache.state,
+                             items, self.num_heads, "additive", max_item_rows=1 if ctx.all_single else 0)
         y = K.gated_group_norm(o, gate, self.gain, self.num_heads, self.eps, self.dtype)
         return K.gemm(y, self.w_out, residual=residual32, out_f32=True, out_scale=self.out_scale)

@@ -195,6 +195,53 @@ def test_retention_scan_with_constant_gates(heads, kd, vd):
         check(state[2], S.numpy(), torch.float32, "final state", loosen=3.0)
 
 
+@pytest.mark.parametrize("heads,kd,vd", [(2, 12, 20), (1, 5, 18), (4, 64, 16), (3, 32, 64), (2, 128, 40), (1, 200, 33),
+                                         (4, 64, 128)])
+def test_retention_in_chunks(heads, kd, vd):
+    """The chunked kernels against the recurrence written out: unequal items in one launch (longer than a chunk, a
+    chunk exactly, one row, a chunk and one row), an item that is skipped, states that are not zero, a request cut
+    into portions at and off the chunks' borders, a decay of one and a fast one."""
+    from swifttransformer_amd.ops import kernels as K
+    g = torch.Generator().manual_seed(3 * kd + vd)
+    decay = [1.0, 0.5, 0.97, 0.9990234375][:heads]
+    lens = [200, 64, 1, 65, 0, 130]
+    slots = [3, 0, 5, 1, -1, 4]
+    T = sum(lens)
+    q, k, v = (torch.randn(T, heads * n, generator=g) for n in (kd, kd, vd))
+    start = torch.randn(6, heads, kd, vd, generator=g)
+    ref = torch.zeros(T, heads, vd, dtype=F64)
+    S = start.to(F64).clone()
+    t0 = 0
+    for n, slot in zip(lens, slots):
+        for h in range(heads):
+            for t in range(t0, t0 + n):
+                S[slot, h] = decay[h] * S[slot, h] + torch.outer(k[t, h * kd:(h + 1) * kd].to(F64) * kd ** -0.5,
+                                                                 v[t, h * vd:(h + 1) * vd].to(F64))
+                ref[t, h] = S[slot, h].T @ q[t, h * kd:(h + 1) * kd].to(F64)
+        t0 += n
+    ref = ref.reshape(T, heads * vd).numpy()
+    decays = torch.tensor(decay, dtype=torch.float32, device=DEV)
+    state = dev(start).clone()
+    # q, k, v as columns of one wider tensor, as the mixer's product leaves them
+    wide = torch.cat([q, k, v], dim=1).to(DEV)
+    qk = heads * kd
+    out = K.retention_chunks(wide[:, :qk], wide[:, qk:2 * qk], wide[:, 2 * qk:], decays, kd ** -0.5, state,
+                             items_ctx(lens, slots), heads)
+    check(out, ref, torch.float32, "items of unequal lengths", loosen=3.0)
+    check(state, S.numpy(), torch.float32, "states after the launch", loosen=3.0)
+    # one request in portions: every cut gives the recurrence's values
+    n0 = lens[0]
+    for cuts in ([n0], [64, 64, 72], [3, 61, 1, 70, 65]):
+        state = dev(start).clone()
+        outs, t0 = [], 0
+        for n in cuts:
+            outs.append(K.retention_chunks(dev(q[t0:t0 + n]), dev(k[t0:t0 + n]), dev(v[t0:t0 + n]), decays, kd ** -0.5,
+                                           state, items_ctx([n], [3]), heads))
+            t0 += n
+        check(torch.cat(outs), ref[:n0], torch.float32, f"portions {cuts}", loosen=3.0)
+        check(state[3], S[3].numpy(), torch.float32, f"state after portions {cuts}", loosen=3.0)
+
+
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("T,E,top,W,F", [(5, 4, 2, 64, 24), (70, 3, 3, 72, 20), (9, 5, 1, 72, 50), (700, 8, 2, 128, 40)])
 def test_experts_weighted_by_the_softmax_over_the_chosen(dtype, T, E, top, W, F):
@@ -441,6 +488,28 @@ def test_the_step_that_is_recorded_gives_its_own_result_also_where_its_tensors_l
     runner.arena.resize(256)
     run_schedule(runner, seqs, refs, [[(0, 70)], [(1, 66)], [(0, 70)], [(1, 66)]], dtype, f"{dtype} outside the arena")
     assert runner.arena.overflows > 0 and runner.graph_replays == 3
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("name", list(tiny.CONFIGS))
+def test_long_portions_take_the_chunked_retention_and_short_ones_the_scan_on_one_state(models, name, dtype, monkeypatch):
+    folder, cfg, w = models[name]
+    seq = tiny.prompt(150, cfg["vocab"], 7)
+    ref = plain.logits(cfg, w, seq).numpy()
+    ps = tiny.PAGE_SIZE[name]
+    runner = make_runner(folder, dtype, ps, -(-150 // ps) + 2, record_after=2)
+    what = f"{name} {dtype}"
+    run_schedule(runner, {0: seq}, {0: ref}, [[(0, 150)]], dtype, what + " whole", loosen=2.0)
+    run_schedule(runner, {0: seq}, {0: ref}, [[(0, 100)]] + [[(0, 1)]] * 50, dtype, what + " decoded", loosen=2.0)
+    run_schedule(runner, {0: seq}, {0: ref}, [[(0, n)] for n in (70, 3, 64, 13)], dtype, what + " portions", loosen=2.0)
+    # every step with a portion in chunks, down to two rows, beside single tokens of another request
+    from swifttransformer_amd.parts.retention import Retention
+    monkeypatch.setattr(Retention, "chunked_from", 2)
+    other = tiny.prompt(30, cfg["vocab"], 8)
+    refs = {0: ref, 1: plain.logits(cfg, w, other).numpy()}
+    runner = make_runner(folder, dtype, ps, -(-150 // ps) + -(-30 // ps) + 2, record_after=2)
+    schedule = [[(0, 2), (1, 20)], [(1, 1), (0, 65)], [(0, 3), (1, 1)], [(1, 1), (0, 64)], [(0, 16), (1, 7)]]
+    run_schedule(runner, {0: seq, 1: other}, refs, schedule, dtype, what + " mixed", loosen=2.0)
 
 
 def test_greedy_generation_through_the_engine(models):
