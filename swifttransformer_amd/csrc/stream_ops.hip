@@ -14,7 +14,7 @@
 //                  small products, the activation, the norm and the sum in one kernel.
 //
 // Everything is float except the optional copy of the dynamic tanh in the storage type and the token side
-// input's two products, whose operands are of the storage type (sums in float).
+// input's matrices and table, which are of the storage type.
 #include "activation.h"
 #include "api.h"
 #include "common.h"
@@ -67,14 +67,12 @@ __global__ __launch_bounds__(256) void row_add_kernel(float* __restrict__ out, c
     out[idx] = v + vec[idx % width];
 }
 
-template <typename T> __device__ inline float as_stored(float v);
-template <> __device__ inline float as_stored<float>(float v) { return v; }
-template <> __device__ inline float as_stored<bf16_t>(float v) { return bf16_to_float(float_to_bf16(v)); }
-
 // A workgroup a row: 16 waves where rows are few (a decode step: every gate feature's row of G in flight
-// at once, the kernel's time a handful of dependent trips to memory), 4 otherwise.  LDS: the row in the
-// storage type's values (as floats), later the projection's result; the gated vector.
-// g_j = stored(gelu(stored(G_j . x)) * e_j), y = P g, x += y / sqrt(mean(y^2) + eps) * w.
+// at once, the kernel's time a handful of dependent trips to memory), 4 otherwise.  LDS: the float row,
+// later the projection's result; the gated vector.  Only the matrices and the table are of the storage
+// type: the row, the gate's sums and the gated vector stay float (a unit norm follows, and a gated vector
+// of a few entries near zero would turn a rounding into a direction).
+// g_j = gelu(G_j . x) * e_j, y = P g, x += y / sqrt(mean(y^2) + eps) * w.
 // VEC: rows of G and P allow 16-byte loads.
 template <typename T, bool VEC>
 __global__ __launch_bounds__(1024) void token_side_kernel(
@@ -96,7 +94,7 @@ __global__ __launch_bounds__(1024) void token_side_kernel(
     const T* er = table + (int64_t)(known ? tok : 0) * table_stride;
     // the first feature's table entry is asked for before the row arrives
     float e = (known && wave < dim) ? Elem<T>::load(er + wave) : 0.f;
-    for (int c = threadIdx.x; c < width; c += threads) xs[c] = as_stored<T>(xr[c]);
+    for (int c = threadIdx.x; c < width; c += threads) xs[c] = xr[c];
     __syncthreads();
     for (int j = wave; j < dim; j += waves) {
         const T* gr = w_gate + (int64_t)j * width;
@@ -112,7 +110,7 @@ __global__ __launch_bounds__(1024) void token_side_kernel(
             for (int c = lane; c < width; c += 64) acc = fmaf(Elem<T>::load(gr + c), xs[c], acc);
         }
         acc = wave_sum(acc);
-        if (lane == 0) gs[j] = as_stored<T>(apply_activation(kActGeluTanh, as_stored<T>(acc)) * e);
+        if (lane == 0) gs[j] = apply_activation(kActGeluTanh, acc) * e;
         if (j + waves < dim) e = known ? Elem<T>::load(er + j + waves) : 0.f;
     }
     __syncthreads();                      // every wave has read xs; gs is complete

@@ -1350,8 +1350,8 @@ def token_side(x: torch.Tensor, token_ids: torch.Tensor, token_item: Optional[to
                w_gate: torch.Tensor, w_proj: torch.Tensor, gain: torch.Tensor, eps: float) -> torch.Tensor:
     """x[t] += unit(w_proj (gelu_tanh(w_gate x[t]) * table[token_ids[t]])) * gain, in place on the float rows x
     [T, width]; unit(y) = y / sqrt(mean(y^2) + eps).  table [vocab, dim] (rows may be strided: columns of a wider
-    table), w_gate [dim, width], w_proj [width, dim] of one storage type: the two products take operands of that
-    type (x rounded to it) and sum in float.  Rows with token_item < 0 are left alone."""
+    table), w_gate [dim, width], w_proj [width, dim] of one storage type; the row, the sums and the gated vector are
+    float.  Rows with token_item < 0 are left alone."""
     T, W = x.shape
     dim = w_gate.shape[0]
     _need(x, "x", torch.float32, (T, W))

@@ -4,8 +4,8 @@ stream and re-enters it at unit root mean square.
     e = E[token, index * dim : (index + 1) * dim]         one table for all layers, a part of a row a layer
     g = gelu_tanh(G x) * e;  y = P g;  x <- x + y / rms(y) * s
 
-The two products take the engine's storage type (sums in float); the unit norm and the sum into the stream
-are float.  One kernel a row does all of it (``token_side``: the row in LDS, a wave a gate feature, a thread
+The two matrices and the table are of the engine's storage type; the stream's row, the sums, the gated
+vector, the unit norm and the sum into the stream are float.  One kernel a row does all of it (``token_side``: the row in LDS, a wave a gate feature, a thread
 an output feature); a stream wider than that kernel's LDS takes the separate kernels.  The reference has
 no such part."""
 from __future__ import annotations

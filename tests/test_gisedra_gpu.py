@@ -105,8 +105,7 @@ def test_token_side_input_in_one_kernel(dtype, W, dim, parts, index):
                f"l{index}.side.gate": rounded(torch.randn(dim, W, generator=g) / W ** 0.5, dtype),
                f"l{index}.side.proj": rounded(torch.randn(W, dim, generator=g) / dim ** 0.5, dtype),
                f"l{index}.side.norm": 0.5 + 0.1 * torch.randn(W, generator=g).to(F64)}
-    xs = rounded(x, dtype)                      # the products read the stream in the storage type
-    ref = x.to(F64) + plain.side_input(xs, tokens, weights, index, dim, eps)
+    ref = x.to(F64) + plain.side_input(x.to(F64), tokens, weights, index, dim, eps)
     ref[4] = x[4].to(F64)                       # a padding row stays as it is
     item = torch.zeros(T, dtype=torch.int32)
     item[4] = -1
