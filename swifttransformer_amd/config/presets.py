@@ -153,3 +153,48 @@ def gisedra_preset(name: str, **overrides):
                         max_positions=4096)
     fields.update(overrides)
     return GisedraHyperParam(**fields).validate()
+
+
+# ---- named sizes of the Pupalix family, for runs with random weights: the layer sizes of the OPT model of the
+# same name.  Of every four layers the first is latent attention (dense gated feed-forward), the second grouped
+# attention whose values are its keys (chunks of 1,024 positions, a quarter of the heads as key heads, routed
+# experts), the third and fourth lightning attention (dense, then routed); four streams; the first two layers
+# run twice.
+def pupalix_preset(name: str, **overrides):
+    from .pupalix_param import PupalixHyperParam
+    key = name.lower().replace("-", "_")
+    size = key.split("_", 1)[1] if "_" in key else ""
+    if "opt_" + size not in _SIZES:
+        raise KeyError(f"invalid model name {name!r}; valid names: " +
+                       " ".join("pupalix_" + k.split("_", 1)[1] for k in _SIZES))
+    n_layers, hidden, heads, ffn = _SIZES["opt_" + size]
+    n_layers = int(overrides.pop("num_layers", n_layers))
+    only = overrides.pop("only", None)            # one mixer type for every layer (measurements)
+    chunk = int(overrides.pop("chunk", 1024))
+    loop_times = int(overrides.pop("loop_times", 2))
+    hd = hidden // heads
+    layers = []
+    for i in range(n_layers):
+        kind = only or ("latent_attention", "attention", "lightning", "lightning")[i % 4]
+        if kind == "latent_attention":
+            mixer = {"heads": heads, "dim": hd, "rot_dim": 32, "vdim": hd, "kv_rank": 128, "scale": float(hd + 32) ** -0.5,
+                     "rot": {"base": 10000.0, "dims": 32,
+                             "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+        elif kind == "attention":
+            mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": hd, "vdim": hd, "scale": float(hd) ** -0.5,
+                     "softcap": 30.0, "mask": {"size": chunk}}
+        else:
+            lh = max(1, heads // 8)
+            mixer = {"heads": lh, "dim": hd, "vdim": 2 * hd, "decay": [1.0 - 2.0 ** (-5 - (j % 4)) for j in range(lh)]}
+        if i % 2 == 0:
+            mlp = {"kind": "dense", "ff": ffn // 2}
+        else:
+            mlp = {"kind": "moe", "router": {"experts": 16, "top": 2, "groups": {"count": 4, "keep": 2}},
+                   "expert": {"ff": ffn // 4}}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    loop = {"start": 0, "stop": min(2, n_layers), "times": loop_times} if loop_times > 0 else None
+    fields: Dict = dict(vocab=50272, width=hidden, layers=layers, loop=loop, streams=4, embedding_scale=float(hidden) ** 0.5,
+                        bigram={"buckets": 65521, "mul_prev": 36313, "mul_cur": 27191}, logit_scale=1.0,
+                        logit_softcap=30.0, norm_eps=1e-5, max_positions=4096)
+    fields.update(overrides)
+    return PupalixHyperParam(**fields).validate()

@@ -57,7 +57,7 @@ def registered_architectures():
 
 def _ensure_builtin() -> None:
     # the built-in architectures register themselves on import
-    from ..models import opt, zitupel, zimorax, gisedra  # noqa: F401
+    from ..models import opt, zitupel, zimorax, gisedra, pupalix  # noqa: F401
 
 
 def resolve_architecture(name: str) -> Architecture:

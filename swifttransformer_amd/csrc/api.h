@@ -53,12 +53,15 @@ int st_gemm_wide_offered(int M, int N, int K, int dtype);
 int st_gemm_wide_groups();
 int st_gemm_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim, int dtype);
 
+// window > 0: a row reads the last `window` positions; window < 0: the positions of its own chunk of -window
+// positions, chunks counted from the sequence's first position; softcap > 0: scaled scores pass through
+// softcap * tanh(score / softcap) before the softmax.  The same for st_attn_prefill.
 int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
                  const void* k_cache, const void* v_cache, int64_t page_stride,
                  const int* row_ids, const int* token_item, const int* positions,
                  const int* block_table, const float* head_slopes,
                  int max_pages, int page_size, int num_tokens, int num_q_heads,
-                 int num_kv_heads, int head_dim, float scale, int window, int num_splits,
+                 int num_kv_heads, int head_dim, float scale, int window, float softcap, int num_splits,
                  int num_waves, int dtype, hipStream_t stream);
 
 // No counterpart in the reference.  For callers that cannot allocate (code under HIP graph
@@ -83,7 +86,7 @@ int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const int* tile_item, const int* tile_q0, int num_tiles,
                     const int* item_tok_off, const int* item_start, const int* item_len,
                     const int* block_table, const float* head_slopes, int max_pages, int page_size,
-                    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, float softcap,
                     int key_split, int tile_rows, int algo, int dtype, hipStream_t stream);
 
 int st_has_attn_prefill();
@@ -153,11 +156,12 @@ int st_state_scan(float* out, const float* q, int64_t q_stride, const float* k, 
                   int64_t slot_stride, const int* item_len, const int* item_tok_off, const int* item_slot,
                   int num_items, int max_item_rows, int heads, int qk_heads, int key_dim, int value_dim, int mode,
                   hipStream_t stream);
-// out = val * rsqrt(mean(val^2) + eps) * gain (* silu(gate) unless gate_first) over each of `groups`
-// parts of a row, val = o (* silu(gate) if gate_first); gain [width], or [groups * width] if gain_per_group.
+// out = val * rsqrt(mean(val^2) + eps) * gain (* act(gate) unless gate_first) over each of `groups`
+// parts of a row, val = o (* act(gate) if gate_first); gain [width], or [groups * width] if gain_per_group;
+// act: silu (gate_kind 0) or sigmoid (gate_kind 1).
 int st_gated_group_norm(void* out, const float* o, const void* gate, int64_t gate_stride, const float* gain,
-                        int num_tokens, int groups, int width, int gain_per_group, int gate_first, float eps,
-                        int dtype, hipStream_t stream);
+                        int num_tokens, int groups, int width, int gain_per_group, int gate_first, int gate_kind,
+                        float eps, int dtype, hipStream_t stream);
 
 // ---- retention in chunks (csrc/retention.hip): S <- decay_h S + (key_factor k) v^T, o = S^T q over each item's rows,
 // from and back to the item's state slot, as products within chunks of st_retention_chunk_rows(key_dim) rows and a
@@ -196,18 +200,21 @@ int st_gated_head_norm(void* out, const float* o, int parts, int64_t part_stride
 // gain, and stored as the token's entry of a one-head page pool whose entries are `entry` >= rank
 // wide (the rest is cleared): [pages, 1, page_size, entry] of `dtype`.  tail > 0: the row's next `tail`
 // values follow the latent in the entry as they are, or, with `freq` [tail / 2], turned by the token's
-// position (pairs 2i, 2i + 1; angle position * freq[i]): a key part that every head shares.
+// position (pairs 2i, 2i + 1; angle position * freq[i]; cosine and sine times tail_mult): a key part that every
+// head shares.
 int st_latent_write(void* cache, int64_t page_stride, const float* x, int64_t x_stride, const float* gain,
                     const int* token_item, const int* positions, const int* block_table, int max_pages,
                     int page_size, int num_tokens, int rank, int entry, float eps, int tail, const float* freq,
-                    int dtype, hipStream_t stream);
+                    float tail_mult, int dtype, hipStream_t stream);
 
 // ---- routed experts (csrc/moe.hip)
 // ids[t, j], weights[t, j] (j < top): the experts with the largest logits of row t, largest first,
 // the lower index on ties, and their weights: mode 0 the sigmoid of each logit, mode 1 the softmax over
-// the chosen logits alone.  Rows whose item is -1 get ids of -1.
+// the chosen logits alone, mode 2 each chosen expert's share of the softmax over all experts, where only the
+// experts of the `keep` best of `groups` equal groups of neighbours (a group's rank: its largest logit) can be
+// chosen.  Rows whose item is -1 get ids of -1.
 int st_moe_route(int* ids, float* weights, const float* logits, const int* token_item, int num_tokens,
-                 int experts, int top, int mode, hipStream_t stream);
+                 int experts, int top, int mode, int groups, int keep, hipStream_t stream);
 // Sorts the num_pairs = tokens * top (token, choice) pairs by expert into tiles of `tile` (16, 64 or 128)
 // places that hold one expert's pairs each: sorted[capacity] (pair index, or -1),
 // place_of_pair[num_pairs] (or -1), tile_expert[capacity / tile] (or -1).
@@ -251,6 +258,31 @@ int st_row_add(float* out, const float* x, const float* first, const float* vec,
 int st_token_side(float* x, const int* token_ids, const int* token_item, const void* table, int64_t table_stride,
                   int vocab, const void* w_gate, const void* w_proj, const float* gain, int num_rows, int dim,
                   int width, float eps, int dtype, hipStream_t stream);
+
+// x[i] = cap * tanh(x[i] * scale / cap) over n floats in place (cap <= 0: x[i] * scale).
+int st_scale_softcap(float* x, int64_t n, float scale, float cap, hipStream_t stream);
+
+// ---- a residual stream of several copies (csrc/hyper_streams.hip); x float [rows, streams, width]
+int st_streams_expand(float* out, const float* x, int num_rows, int streams, int width, hipStream_t stream);
+int st_streams_sum(float* out, const float* x, const int* rows, int num_rows, int streams, int width,
+                   hipStream_t stream);
+int st_streams_read(void* out_t, float* out32, const float* x, const float* a, const float* gain, int num_rows,
+                    int streams, int width, float eps, int dtype, hipStream_t stream);
+int st_streams_write(float* x, const float* y, const float* mix, const float* b, void* out_t, const float* a2,
+                     const float* gain2, int num_rows, int streams, int width, float eps2, int dtype,
+                     hipStream_t stream);
+
+// ---- token embedding times a factor plus a row chosen by a hash of the token and the one before (csrc/hashed_embedding.hip)
+int st_hashed_embed(float* out, const int* ids, const int* positions, const int* token_item, const int* item_len,
+                    const int* item_tok_off, const int* item_slot, int* last_token, const void* table,
+                    const void* pairs, int num_tokens, int num_items, int vocab, int buckets, int64_t mul_prev,
+                    int64_t mul_cur, float scale, int width, int dtype, hipStream_t stream);
+
+// ---- queries and keys normalised over their whole projection, the keys as projected as values (csrc/tied_attention.hip)
+int st_qk_norm_write(void* out_q, void* k_cache, void* v_cache, int64_t page_stride, const float* qk, int64_t stride,
+                     const float* gain_q, const float* gain_k, const int* token_item, const int* positions,
+                     const int* block_table, int max_pages, int page_size, int num_tokens, int heads, int kv_heads,
+                     int head_dim, int head_pad, float eps, int write, int dtype, hipStream_t stream);
 
 // Measurement kernels (csrc/probe.hip): a plain streaming read, and a kernel without work.
 int st_probe_read(const void* src, int64_t bytes, void* sink, int workgroups, int pattern, hipStream_t stream);

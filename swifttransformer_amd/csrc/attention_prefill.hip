@@ -7,7 +7,7 @@
 // longest chain of dependent key blocks, which is what bounds the kernel when few tiles are
 // in flight: a late tile of a long prompt, or a portion that attends to a long cache.  The portion's own keys and values are already
 // in the cache, so the keys of a row at position p are simply the cached positions
-// [lo, p] of its request (lo > 0 only with a window), read through the block table in
+// [lo, p] of its request (lo > 0 only with a window or with chunks), read through the block table in
 // blocks of 64 keys that all four waves share through LDS.  Softmax is online in float;
 // both products accumulate in float.
 //
@@ -58,8 +58,8 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
     const int* __restrict__ block_table, const float* __restrict__ head_slopes, int max_pages, int page_size,
-    int page_shift, int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_tiles,
-    int deal_period) {
+    int page_shift, int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, float softcap,
+    int num_tiles, int deal_period) {
     constexpr int KS_STRIDE = 32 * HDP + 8;          // elements between keys of the K block
     extern __shared__ uint4 dyn[];
     constexpr int BUF = PK * KS_STRIDE + (32 * HDP) * VT_STRIDE;   // elements of the block buffer
@@ -92,7 +92,12 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
     // keys needed by the tile
     const int rows_in_tile = min(PQ, n - q0);
     const int pos_first = start + q0, pos_last = start + q0 + rows_in_tile - 1;
-    const int key_lo = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+    // window > 0: a row sees the last `window` positions; window < 0: the positions of its own chunk of -window
+    // positions (chunks counted from the sequence's start)
+    const int csize = window < 0 ? -window : 0;
+    const int key_lo = window > 0 ? (pos_first + 1 > window ? pos_first + 1 - window : 0)
+                                  : csize ? pos_first - pos_first % csize : 0;
+    const int row_lo = window > 0 ? qpos - window + 1 : csize ? qpos - qpos % csize : 0;   // this lane's row
     const int key_hi = pos_last + 1;                 // exclusive
 
     // block table of the request -> LDS
@@ -221,7 +226,10 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
     // scores.  The scores of such a head are turned into their final log2 units right after the
     // product (c = 1 from then on); all others stay raw and are scaled inside the exponential.
     const float bias_l2 = head_slopes ? head_slopes[h] * 1.44269504088896340736f : 0.f;
-    const bool biased = bias_l2 != 0.f;
+    // capped scores, cap * tanh(s / cap), are made final in the same place
+    const bool capped = softcap > 0.f;
+    const float inv_cap = capped ? scale / softcap : 0.f, cap_l2 = softcap * 1.44269504088896340736f;
+    const bool biased = bias_l2 != 0.f || capped;
     const float c = biased ? 1.f : sl;
 
     auto consume = [&](int kb, int buf) {
@@ -251,7 +259,13 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
         // c = scale * log2(e): one multiply-add and one exp2 per score.  Blocks entirely visible
         // to all rows of the wave (the common case away from the diagonal and the window's
         // edge) skip the masking.
-        if (biased) {
+        if (capped) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    st[t][r] = fmaf(cap_l2, tanhf(st[t][r] * inv_cap), bias_l2 * (float)(kb + 16 * t + 4 * g + r - qpos));
+        } else if (biased) {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -259,7 +273,8 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
                     st[t][r] = fmaf(st[t][r], sl, bias_l2 * (float)(kb + 16 * t + 4 * g + r - qpos));
         }
         const bool interior = kb + PK - 1 <= wave_first && kb >= key_lo &&
-                              (window <= 0 || kb > wave_last - window);
+                              (window <= 0 || kb > wave_last - window) &&
+                              (csize == 0 || kb >= wave_last - wave_last % csize);
         float bmax = -INFINITY;
         if (interior) {
 #pragma unroll
@@ -272,7 +287,7 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int j = kb + 16 * t + 4 * g + r;
-                    const bool ok = qvalid && j <= qpos && j >= key_lo && (window <= 0 || j > qpos - window);
+                    const bool ok = qvalid && j <= qpos && j >= key_lo && j >= row_lo;
                     const float sv = ok ? st[t][r] : -INFINITY;
                     st[t][r] = sv;
                     bmax = fmaxf(bmax, sv);
@@ -424,7 +439,7 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
                           int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                           const int* item_tok_off, const int* item_start, const int* item_len,
                           const int* block_table, const float* head_slopes, int max_pages, int page_size,
-                          int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
+                          int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, float softcap,
                           hipStream_t stream) {
     auto kernel = attn_prefill_kernel<HDP, KS>;
     const size_t lds = prefill_lds(HDP, KS, max_pages);
@@ -448,7 +463,7 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
     kernel<<<dim3(num_q_heads, num_tiles), 256 * KS, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
         tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, head_slopes, max_pages, page_size,
-        page_shift, num_q_heads, num_kv_heads, head_dim, scale, window, num_tiles, deal_period);
+        page_shift, num_q_heads, num_kv_heads, head_dim, scale, window, softcap, num_tiles, deal_period);
     ST_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
@@ -471,7 +486,8 @@ int attn_prefill_f32(void* out, const void* q, int64_t q_stride, const void* k_c
                      int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                      const int* item_tok_off, const int* item_start, const int* item_len,
                      const int* block_table, const float* head_slopes, int max_pages, int page_size,
-                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, hipStream_t stream);
+                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, float softcap,
+                     hipStream_t stream);
 
 // the direct-load instance (attention_prefill_dma.hip)
 bool attn_prefill_dma_offered(int head_dim, int page_size, int tile_rows, int max_pages);
@@ -501,7 +517,7 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const int* tile_item, const int* tile_q0, int num_tiles,
                     const int* item_tok_off, const int* item_start, const int* item_len,
                     const int* block_table, const float* head_slopes, int max_pages, int page_size,
-                    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, float softcap,
                     int key_split, int tile_rows, int algo, int dtype, hipStream_t stream) {
     ST_CHECK(dtype == kBF16 || dtype == kF32, "attn_prefill: unknown dtype %d", dtype);
     ST_CHECK(num_tiles >= 0 && num_q_heads > 0 && num_kv_heads > 0 && page_size > 0 && max_pages > 0,
@@ -511,13 +527,13 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
     ST_CHECK(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
              "attn_prefill: head_dim %d is not a multiple of 16 in [16, 256]", head_dim);
     ST_CHECK(num_tiles <= 65535, "attn_prefill: too many tiles for one launch");
-    ST_CHECK(window >= 0, "attn_prefill: negative window");
+    ST_CHECK(softcap >= 0.f && softcap <= 3.0e38f, "attn_prefill: the cap of the scores must be finite and not negative");
     ST_CHECK(scale == scale && scale >= -3.0e38f && scale <= 3.0e38f, "attn_prefill: the score scale must be finite");
     ST_CHECK(tile_rows == 64 || tile_rows == 128, "attn_prefill: tiles of %d rows (64 or 128)", tile_rows);
     ST_CHECK(algo >= 0 && algo <= 2, "attn_prefill: unknown algo %d", algo);
-    // (the direct-load kernel has no score bias: heads with slopes go through the staging kernel)
+    // (the direct-load kernel has no score bias, no cap and no chunks: those go through the staging kernel)
     // (and it orders maxima in scaled units, which needs a positive, finite scale)
-    const bool dma_ok = dtype == kBF16 && !head_slopes && scale > 0.f && scale <= 3.0e38f &&
+    const bool dma_ok = dtype == kBF16 && !head_slopes && softcap == 0.f && window >= 0 && scale > 0.f && scale <= 3.0e38f &&
                         attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages);
     ST_CHECK(tile_rows == 64 || (dma_ok && algo != 1),
              "attn_prefill: tiles of 128 rows need the direct-load kernel (bfloat16, head_dim 64 or 128, "
@@ -529,7 +545,7 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
     if (dtype == kF32)
         return attn_prefill_f32(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles,
                                 item_tok_off, item_start, item_len, block_table, head_slopes, max_pages, page_size,
-                                num_q_heads, num_kv_heads, head_dim, scale, window, stream);
+                                num_q_heads, num_kv_heads, head_dim, scale, window, softcap, stream);
     ST_CHECK(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
     const int hdp = (head_dim + 31) / 32;
     // the direct-load kernel wherever it is offered
@@ -544,7 +560,7 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
              "attn_prefill: %d wave groups are not offered for head_dim %d", ks, head_dim);
 #define ST_PF(H, S) launch_prefill<H, S>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles, \
         item_tok_off, item_start, item_len, block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, \
-        head_dim, scale, window, stream)
+        head_dim, scale, window, softcap, stream)
     switch (hdp * 8 + ks) {
         case 1 * 8 + 1: return ST_PF(1, 1);
         case 1 * 8 + 2: return ST_PF(1, 2);

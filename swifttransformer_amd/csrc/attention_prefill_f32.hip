@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
     const int* __restrict__ block_table, const float* __restrict__ head_slopes, int max_pages, int page_size,
-    int num_q_heads, int num_kv_heads, float scale, int window, int num_tiles, int deal_period) {
+    int num_q_heads, int num_kv_heads, float scale, int window, float softcap, int num_tiles, int deal_period) {
     constexpr int HD = 16 * DT;
     constexpr int K_STRIDE = HD + 4;                 // floats between keys of the K block
     extern __shared__ uint4 dyn[];
@@ -68,7 +68,13 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     const int qpos = start + qi;
     const int rows_in_tile = min(PQ, n - q0);
     const int pos_first = start + q0, pos_last = start + q0 + rows_in_tile - 1;
-    const int key_lo = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+    // window > 0: a row sees the last `window` positions; window < 0: the positions of its own chunk of -window
+    // positions (chunks counted from the sequence's start)
+    const int csize = window < 0 ? -window : 0;
+    const int key_lo = window > 0 ? (pos_first + 1 > window ? pos_first + 1 - window : 0)
+                                  : csize ? pos_first - pos_first % csize : 0;
+    const int row_lo = window > 0 ? qpos - window + 1 : csize ? qpos - qpos % csize : 0;   // this lane's row
+    const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;   // scores pass through softcap * tanh(s / softcap)
     const int key_hi = pos_last + 1;                 // exclusive
 
     {
@@ -148,8 +154,10 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int j = kb + 16 * t + 4 * g + r;
-                const bool ok = qvalid && j <= qpos && j >= key_lo && (window <= 0 || j > qpos - window);
-                const float s = ok ? fmaf(slope, (float)(j - qpos), st[t][r] * scale) : -INFINITY;   // slope 0: the score itself
+                const bool ok = qvalid && j <= qpos && j >= key_lo && j >= row_lo;
+                float sc = st[t][r] * scale;
+                if (softcap > 0.f) sc = softcap * tanhf(sc * inv_cap);
+                const float s = ok ? fmaf(slope, (float)(j - qpos), sc) : -INFINITY;   // slope 0: the score itself
                 st[t][r] = s;
                 bmax = fmaxf(bmax, s);
             }
@@ -213,7 +221,7 @@ int launch(float* out, const float* q, int64_t q_stride, const float* k_cache, c
            int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
            const int* item_tok_off, const int* item_start, const int* item_len, const int* block_table,
            const float* head_slopes, int max_pages, int page_size, int num_q_heads, int num_kv_heads, float scale,
-           int window, hipStream_t stream) {
+           int window, float softcap, hipStream_t stream) {
     constexpr int HD = 16 * DT;
     auto kernel = attn_prefill_f32_kernel<DT>;
     const size_t lds = (size_t)(PK * (HD + 4) + HD * VT_STRIDE) * sizeof(float) + (size_t)max_pages * sizeof(int);
@@ -233,8 +241,8 @@ int launch(float* out, const float* q, int64_t q_stride, const float* k_cache, c
     const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
     kernel<<<dim3(num_q_heads, num_tiles), 256, lds, stream>>>(
         out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, item_tok_off, item_start, item_len,
-        block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, num_tiles,
-        deal_period);
+        block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, softcap,
+        num_tiles, deal_period);
     ST_LAUNCH_CHECK("attn_prefill (float)");
     return 0;
 }
@@ -246,11 +254,12 @@ int attn_prefill_f32(void* out, const void* q, int64_t q_stride, const void* k_c
                      int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                      const int* item_tok_off, const int* item_start, const int* item_len,
                      const int* block_table, const float* head_slopes, int max_pages, int page_size,
-                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, hipStream_t stream) {
+                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, float softcap,
+                     hipStream_t stream) {
     ST_CHECK(q_stride % 4 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
 #define ST_PF(D) case D: return launch<D>((float*)out, (const float*)q, q_stride, (const float*)k_cache,          \
         (const float*)v_cache, page_stride, tile_item, tile_q0, num_tiles, item_tok_off, item_start, item_len,    \
-        block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, stream)
+        block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, softcap, stream)
     switch (head_dim / 16) {
         ST_PF(1); ST_PF(2); ST_PF(3); ST_PF(4); ST_PF(5); ST_PF(6); ST_PF(7); ST_PF(8);
         ST_PF(9); ST_PF(10); ST_PF(11); ST_PF(12); ST_PF(13); ST_PF(14); ST_PF(15); ST_PF(16);

@@ -103,7 +103,7 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, int64_t page_stride,
     const int* __restrict__ row_ids, const int* __restrict__ token_item, const int* __restrict__ positions,
     const int* __restrict__ block_table, const float* __restrict__ head_slopes, int max_pages, int page_size,
-    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_splits) {
+    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, float softcap, int num_splits) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int KPW = kWave / LPK;        // keys per wave per step
     const int G = (blockDim.x >> 6) * KPW;  // lane groups in the workgroup (4 or 8 waves)
@@ -129,7 +129,9 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
     int kb = 0, ke = 0;
     if (item >= 0 && pos >= 0) {
         const int hi = pos + 1;
-        const int lo = (window > 0 && hi > window) ? hi - window : 0;
+        // window > 0: the last `window` positions; window < 0: the positions of the row's own chunk of
+        // -window positions, chunks counted from the sequence's start
+        const int lo = window > 0 ? (hi > window ? hi - window : 0) : window < 0 ? pos - pos % (-window) : 0;
         const int chunk = (hi - lo + num_splits - 1) / num_splits;
         kb = lo + split * chunk;
         ke = min(hi, kb + chunk);
@@ -165,6 +167,7 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
     const int64_t head_off = (int64_t)kvh * page_size * head_dim + d0;
     // a position encoding may add slope * (key position - query position) to this head's scores
     const float slope = head_slopes ? head_slopes[h] : 0.f;
+    const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;   // scores pass through softcap * tanh(s / softcap)
     __syncthreads();
 
     float m = -INFINITY, l = 0.f, acc[VEC];
@@ -213,6 +216,7 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             s[u] = fmaf(slope, (float)(j0 + u * G - pos), group_sum<LPK>(s[u]) * post_scale);   // slope 0: the score itself
+            if (softcap > 0.f) s[u] = softcap * tanhf(s[u] * inv_cap);
             if (j0 + u * G >= ke) s[u] = -INFINITY;      // the same for all lanes of a group
             mn = fmaxf(mn, s[u]);
         }
@@ -324,7 +328,7 @@ static int launch_rows(void* out, float* part_o, float* part_lse, const void* q,
                        const int* row_ids, const int* token_item, const int* positions,
                        const int* block_table, const float* head_slopes,
                        int max_pages, int page_size, int num_tokens, int num_q_heads,
-                       int num_kv_heads, int head_dim, float scale, int window, int num_splits,
+                       int num_kv_heads, int head_dim, float scale, int window, float softcap, int num_splits,
                        int num_waves, hipStream_t stream) {
     constexpr int VEC = Elem<T>::kVec;
     const int need = (head_dim + VEC - 1) / VEC;
@@ -339,7 +343,7 @@ static int launch_rows(void* out, float* part_o, float* part_lse, const void* q,
     attn_rows_kernel<T, L><<<grid, num_waves * 64, lds, stream>>>((T*)out, part_o, part_lse, (const T*)q,  \
         q_stride, (const T*)k_cache, (const T*)v_cache, page_stride, row_ids, token_item, positions, \
         block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, scale, window, \
-        num_splits)
+        softcap, num_splits)
     switch (lpk) {
         case 1: ST_ROWS(1); break;
         case 2: ST_ROWS(2); break;
@@ -378,7 +382,7 @@ extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const voi
                             const int* row_ids, const int* token_item, const int* positions,
                             const int* block_table, const float* head_slopes,
                             int max_pages, int page_size, int num_tokens, int num_q_heads,
-                            int num_kv_heads, int head_dim, float scale, int window, int num_splits,
+                            int num_kv_heads, int head_dim, float scale, int window, float softcap, int num_splits,
                             int num_waves, int dtype, hipStream_t stream) {
     ST_CHECK(num_tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0 && page_size > 0 &&
              max_pages > 0, "attention: bad sizes");
@@ -389,17 +393,17 @@ extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const voi
     ST_CHECK(num_tokens <= 65535, "attention: more than 65535 rows in one launch");
     ST_CHECK(num_splits == 1 || (part_o && part_lse), "attention: split needs partial buffers");
     ST_CHECK(out || num_splits > 1, "attention: no destination");
-    ST_CHECK(window >= 0, "attention: negative window");
+    ST_CHECK(softcap >= 0.f && softcap <= 3.0e38f, "attention: the cap of the scores must be finite and not negative");
     ST_CHECK(num_waves == 4 || num_waves == 8, "attention: %d waves per workgroup (4 or 8)", num_waves);
     if (num_tokens == 0) return 0;
     if (dtype == kF32)
         return launch_rows<float>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
                                   row_ids, token_item, positions, block_table, head_slopes, max_pages, page_size, num_tokens,
-                                  num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, num_waves, stream);
+                                  num_q_heads, num_kv_heads, head_dim, scale, window, softcap, num_splits, num_waves, stream);
     if (dtype == kBF16)
         return launch_rows<bf16_t>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
                                    row_ids, token_item, positions, block_table, head_slopes, max_pages, page_size, num_tokens,
-                                   num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, num_waves, stream);
+                                   num_q_heads, num_kv_heads, head_dim, scale, window, softcap, num_splits, num_waves, stream);
     ST_CHECK(false, "attention: unknown dtype %d", dtype);
     return 0;
 }
@@ -441,5 +445,5 @@ extern "C" int st_attn_rows_static(void* out, const void* q, int64_t q_stride,
     }
     return st_attn_rows(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride, row_ids,
                         token_item, positions, block_table, head_slopes, max_pages, page_size, num_tokens, num_q_heads,
-                        num_kv_heads, head_dim, scale, window, num_splits, num_waves, dtype, stream);
+                        num_kv_heads, head_dim, scale, window, 0.f, num_splits, num_waves, dtype, stream);
 }

@@ -13,7 +13,7 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
     T* __restrict__ cache, int64_t page_stride, const float* __restrict__ x, int64_t x_stride,
     const float* __restrict__ gain, const int* __restrict__ token_item, const int* __restrict__ positions,
     const int* __restrict__ block_table, int max_pages, int page_size, int num_tokens, int rank, int entry,
-    float eps, int tail, const float* __restrict__ freq) {
+    float eps, int tail, const float* __restrict__ freq, float tail_mult) {
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= num_tokens) return;
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
             if (freq) {                               // pairs (2i, 2i + 1) of the tail turn with the position
                 const int i = (j - rank) >> 1;
                 const float a = (float)pos * freq[i];
-                const float c = cosf(a), s = sinf(a);
+                const float c = cosf(a) * tail_mult, s = sinf(a) * tail_mult;
                 const int ju = rank + 2 * i;
                 const float u = xp[ju], w = xp[ju + 1];
                 v = ((j - rank) & 1) ? w * c + u * s : u * c - w * s;
@@ -53,7 +53,7 @@ using namespace st;
 extern "C" int st_latent_write(void* cache, int64_t page_stride, const float* x, int64_t x_stride, const float* gain,
                                const int* token_item, const int* positions, const int* block_table, int max_pages,
                                int page_size, int num_tokens, int rank, int entry, float eps, int tail,
-                               const float* freq, int dtype, hipStream_t stream) {
+                               const float* freq, float tail_mult, int dtype, hipStream_t stream) {
     ST_CHECK(num_tokens >= 0 && rank > 0 && tail >= 0 && entry >= rank + tail && page_size > 0 && max_pages > 0,
              "latent_write: bad sizes");
     ST_CHECK(!freq || tail % 2 == 0, "latent_write: a turned tail has an even size");
@@ -63,10 +63,10 @@ extern "C" int st_latent_write(void* cache, int64_t page_stride, const float* x,
     const unsigned grid = (unsigned)((num_tokens + 3) / 4);
     if (dtype == kF32)
         latent_write_kernel<float><<<grid, 256, 0, stream>>>((float*)cache, page_stride, x, x_stride, gain, token_item,
-            positions, block_table, max_pages, page_size, num_tokens, rank, entry, eps, tail, freq);
+            positions, block_table, max_pages, page_size, num_tokens, rank, entry, eps, tail, freq, tail_mult);
     else if (dtype == kBF16)
         latent_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)cache, page_stride, x, x_stride, gain, token_item,
-            positions, block_table, max_pages, page_size, num_tokens, rank, entry, eps, tail, freq);
+            positions, block_table, max_pages, page_size, num_tokens, rank, entry, eps, tail, freq, tail_mult);
     else ST_CHECK(false, "latent_write: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("latent_write");
     return 0;

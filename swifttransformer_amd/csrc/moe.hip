@@ -26,7 +26,7 @@ constexpr int kMaxTop = 16;
 
 __global__ __launch_bounds__(256) void moe_route_kernel(
     int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ logits,
-    const int* __restrict__ token_item, int num_tokens, int experts, int top, int mode) {
+    const int* __restrict__ token_item, int num_tokens, int experts, int top, int mode, int groups, int keep) {
     const int t = blockIdx.x * 256 + threadIdx.x;
     if (t >= num_tokens) return;
     if (token_item && token_item[t] < 0) {
@@ -34,12 +34,30 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
         return;
     }
     const float* z = logits + (int64_t)t * experts;
+    // mode 2: only the experts of the `keep` groups (of `groups` equal groups of neighbours) whose largest
+    // logit is largest can be chosen; bit g of `open` says that group g is one of them
+    uint64_t open = ~0ull;
+    const int per = experts / groups;
+    if (mode == 2 && keep < groups) {
+        open = 0;
+        for (int j = 0; j < keep; ++j) {
+            int best = -1;
+            float bv = 0.f;
+            for (int g = 0; g < groups; ++g) {
+                if ((open >> g) & 1) continue;
+                float gv = z[g * per];
+                for (int e = 1; e < per; ++e) gv = fmaxf(gv, z[g * per + e]);
+                if (best < 0 || gv > bv) { best = g; bv = gv; }
+            }
+            open |= 1ull << best;
+        }
+    }
     int chosen[kMaxTop];
     for (int j = 0; j < top; ++j) {
         int best = -1;
         float bv = 0.f;
         for (int e = 0; e < experts; ++e) {
-            bool taken = false;
+            bool taken = mode == 2 && !((open >> (e / per)) & 1);
             for (int u = 0; u < j; ++u) taken |= chosen[u] == e;
             const float v = z[e];
             if (!taken && (best < 0 || v > bv)) { best = e; bv = v; }
@@ -47,6 +65,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
         chosen[j] = best;
         ids[(int64_t)t * top + j] = best;
         weights[(int64_t)t * top + j] = mode == 0 ? 1.f / (1.f + expf(-bv)) : bv;
+    }
+    if (mode == 2) {
+        // the weights are the chosen experts' shares of the softmax over all experts, as they are
+        float m = z[0], sum = 0.f;
+        for (int e = 1; e < experts; ++e) m = fmaxf(m, z[e]);
+        for (int e = 0; e < experts; ++e) sum += expf(z[e] - m);
+        float* w = weights + (int64_t)t * top;
+        for (int j = 0; j < top; ++j) w[j] = expf(w[j] - m) / sum;
     }
     if (mode == 1) {
         // softmax over the chosen logits alone; the first chosen is the largest
@@ -421,15 +447,21 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
 using namespace st;
 
 extern "C" int st_moe_route(int* ids, float* weights, const float* logits, const int* token_item, int num_tokens,
-                            int experts, int top, int mode, hipStream_t stream) {
-    ST_CHECK(mode == 0 || mode == 1, "moe_route: mode 0 (sigmoid of each) or 1 (softmax over the chosen)");
+                            int experts, int top, int mode, int groups, int keep, hipStream_t stream) {
+    ST_CHECK(mode >= 0 && mode <= 2, "moe_route: mode 0 (sigmoid of each), 1 (softmax over the chosen) or 2 (softmax "
+             "over all, the choice within the best groups)");
+    if (mode != 2) groups = keep = 1;
+    ST_CHECK(groups >= 1 && groups <= 64 && experts % groups == 0 && keep >= 1 && keep <= groups,
+             "moe_route: %d experts in %d groups of which %d are kept (up to 64 equal groups)", experts, groups, keep);
+    ST_CHECK(top <= keep * (experts / groups), "moe_route: %d experts a token do not fit %d groups of %d", top, keep,
+             experts / groups);
     ST_CHECK(num_tokens >= 0 && experts > 0, "moe_route: bad sizes");
     ST_CHECK(top >= 1 && top <= kMaxTop && top <= experts, "moe_route: 1 to %d experts a token (of %d), not %d",
              kMaxTop, experts, top);
     ST_CHECK(ids && weights && logits, "moe_route: null operand");
     if (num_tokens == 0) return 0;
     moe_route_kernel<<<(num_tokens + 255) / 256, 256, 0, stream>>>(ids, weights, logits, token_item, num_tokens,
-                                                                  experts, top, mode);
+                                                                  experts, top, mode, groups, keep);
     ST_LAUNCH_CHECK("moe_route");
     return 0;
 }

@@ -262,7 +262,8 @@ __global__ __launch_bounds__(128) void state_scan_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(
     T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ gate, int64_t gate_stride,
-    const float* __restrict__ gain, int groups, int width, int gain_per_group, int gate_first, float eps) {
+    const float* __restrict__ gain, int groups, int width, int gain_per_group, int gate_first, int gate_kind,
+    float eps) {
     __shared__ float red[16];
     const int64_t t = blockIdx.x / groups;
     const int g = blockIdx.x - (int)t * groups;
@@ -275,7 +276,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
         float val = op[j];
         if (gate_first) {
             const float z = Elem<T>::load(gp + j);
-            val *= z / (1.f + expf(-z));
+            val *= (gate_kind ? 1.f : z) / (1.f + expf(-z));
         }
         ss = fmaf(val, val, ss);
     }
@@ -283,7 +284,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
     const float r = 1.f / sqrtf(ss / (float)width + eps);
     for (int j = threadIdx.x; j < width; j += 256) {
         const float z = Elem<T>::load(gp + j);
-        const float s = z / (1.f + expf(-z));
+        const float s = (gate_kind ? 1.f : z) / (1.f + expf(-z));
         const float val = op[j] * r * wp[j] * s;
         Elem<T>::store(dst + j, val);
     }
@@ -364,7 +365,7 @@ extern "C" int st_state_scan(float* out, const float* q, int64_t q_stride, const
 
 extern "C" int st_gated_group_norm(void* out, const float* o, const void* gate, int64_t gate_stride,
                                    const float* gain, int num_tokens, int groups, int width, int gain_per_group,
-                                   int gate_first, float eps, int dtype, hipStream_t stream) {
+                                   int gate_first, int gate_kind, float eps, int dtype, hipStream_t stream) {
     ST_CHECK(num_tokens >= 0 && groups > 0 && width > 0, "gated_group_norm: bad sizes");
     ST_CHECK(eps > 0.f, "gated_group_norm: eps must be positive");
     if (num_tokens == 0) return 0;
@@ -373,10 +374,10 @@ extern "C" int st_gated_group_norm(void* out, const float* o, const void* gate, 
     const unsigned grid = (unsigned)(num_tokens * groups);
     if (dtype == kF32)
         gated_group_norm_kernel<float><<<grid, 256, 0, stream>>>((float*)out, o, (const float*)gate, gate_stride,
-                                                                 gain, groups, width, gain_per_group, gate_first, eps);
+                                                                 gain, groups, width, gain_per_group, gate_first, gate_kind, eps);
     else if (dtype == kBF16)
         gated_group_norm_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, o, (const bf16_t*)gate, gate_stride,
-                                                                  gain, groups, width, gain_per_group, gate_first, eps);
+                                                                  gain, groups, width, gain_per_group, gate_first, gate_kind, eps);
     else ST_CHECK(false, "gated_group_norm: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("gated_group_norm");
     return 0;

@@ -43,6 +43,14 @@ __global__ __launch_bounds__(256) void dynamic_tanh_kernel(
     if (out_t) Elem<T>::store(out_t + idx, y);
 }
 
+// logits through a factor and a smooth limit: cap * tanh(x * scale / cap)
+__global__ __launch_bounds__(256) void scale_softcap_kernel(float* __restrict__ x, int64_t n, float scale, float cap) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i] * scale;
+    x[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+}
+
 // a workgroup a row
 __global__ __launch_bounds__(256) void unit_add_kernel(float* __restrict__ x, const float* __restrict__ y,
                                                        const float* __restrict__ w, int width, float eps) {
@@ -156,6 +164,15 @@ extern "C" int st_dynamic_tanh(void* out_t, float* out32, const float* x, const 
         dynamic_tanh_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out_t, out32, x, rows, w, b, alpha, base, w2, b2, alpha2, width, total);
     else ST_CHECK(false, "dynamic_tanh: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("dynamic_tanh");
+    return 0;
+}
+
+extern "C" int st_scale_softcap(float* x, int64_t n, float scale, float cap, hipStream_t stream) {
+    ST_CHECK(n >= 0 && scale == scale && cap == cap, "scale_softcap: bad operands");
+    if (n == 0) return 0;
+    ST_CHECK(x, "scale_softcap: null operand");
+    scale_softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, n, scale, cap);
+    ST_LAUNCH_CHECK("scale_softcap");
     return 0;
 }
 

@@ -8,6 +8,7 @@ from . import opt  # noqa: F401  (registers OPTForCausalLM)
 from . import zitupel  # noqa: F401  (registers Zitupel)
 from . import zimorax  # noqa: F401  (registers Zimorax)
 from . import gisedra  # noqa: F401  (registers Gisedra)
+from . import pupalix  # noqa: F401  (registers Pupalix)
 from .opt import build_opt_spec
 
 __all__ = ["DecoderModel", "build_opt_spec", "build_model", "load_model", "random_model"]

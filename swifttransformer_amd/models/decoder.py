@@ -32,8 +32,11 @@ class Layer:
     side_input: object = None
 
     def parts(self):
-        return tuple(p for p in (self.mixer_norm, self.mixer_conv, self.mixer, self.mixer_out_norm, self.ffn_norm,
+        return tuple(p for p in (self.arrangement, self.mixer_norm, self.mixer_conv, self.mixer, self.mixer_out_norm, self.ffn_norm,
                                  self.feed_forward, self.ffn_out_norm, self.side_input) if p is not None)
+
+
+EMBEDDING_CACHE = ("embedding",)     # the cache id of what an embedding part keeps a request (its last token)
 
 
 def conv_cache_id(run: int):
@@ -78,6 +81,7 @@ class DecoderModel:
         self.final_norm = build_part("norm", spec.final_norm, H, dtype) if spec.final_norm else None
         self.head = build_part("head", spec.head, H, dtype)
         self.schedule = list(spec.schedule)
+        self.streams = int(getattr(spec, "streams", 0) or 0)
         self.weights_loaded = False
 
     # ------------------------------------------------------------------ weights
@@ -116,6 +120,8 @@ class DecoderModel:
         """cache id -> need, for every cache the schedule writes: the mixers' under the schedule's
         own ids (integers), the state of a run's ``mixer_conv`` part under ``conv_cache_id(run)``."""
         needs: Dict[object, CacheNeed] = {}
+        if hasattr(self.embedding, "cache_need") and self.embedding.cache_need() is not None:
+            needs[EMBEDDING_CACHE] = self.embedding.cache_need()
         for run, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
             if layer.mixer_conv is not None:
@@ -164,11 +170,16 @@ class DecoderModel:
             # the reference refuses to run before weights are loaded (gptop_base.cc:47-49)
             raise RuntimeError("load the weights before running the model")
         ctx.position = self.position
+        embed = ((lambda: self.embedding.forward(ctx, self.position, cache=caches.get(EMBEDDING_CACHE)))
+                 if hasattr(self.embedding, "cache_need") else (lambda: self.embedding.forward(ctx, self.position)))
         if self.entries:
             with K.arena.held():     # read again by the runs that start from it: it lives until the step ends
-                first32 = x32 = self.embedding.forward(ctx, self.position)
+                first32 = x32 = embed()
         else:
-            x32 = self.embedding.forward(ctx, self.position)
+            x32 = embed()
+        if self.streams:
+            with K.arena.held():     # the copies of the stream are updated in place by every layer of the step
+                x32 = K.streams_expand(x32, self.streams)
         for run, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
             K.arena.next_bank()      # what this run of a layer makes may be read until the next one ends
@@ -197,6 +208,8 @@ class DecoderModel:
         if n == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x32.device)
         K.arena.next_bank()
+        if self.streams:             # the final norm reads the sum of the streams, of the wanted rows only
+            x32, rows = K.streams_sum(x32, self.streams, rows), None
         if keep is None:
             keep = not ctx.static_shapes
         takes = getattr(self.head, "takes_norm", None)

@@ -54,11 +54,11 @@ def _lib():
         lib.st_gemm_can_fuse_merge.argtypes = [_c_int] * 7
         lib.st_gemm_library_tuning.argtypes = [_c_int]
         lib.st_attn_rows.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p,
-                                     _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int,
+                                     _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_f, _c_int,
                                      _c_int, _c_int, _c_p]
         lib.st_attn_prefill.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int,
                                         _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                        _c_f, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
+                                        _c_f, _c_int, _c_f, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_attn_prefill_tile_rows.argtypes = [_c_int] * 6
         lib.st_probe_read.argtypes = [_c_p, _c_i64, _c_p, _c_int, _c_int, _c_p]
         lib.st_probe_empty.argtypes = [_c_p, _c_p]
@@ -84,15 +84,15 @@ def _lib():
         lib.st_state_scan.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
                                       _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_gated_group_norm.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                            _c_f, _c_int, _c_p]
+                                            _c_int, _c_f, _c_int, _c_p]
         lib.st_decay_gate.argtypes = [_c_p, _c_p, _c_i64, _c_f, _c_p]
         lib.st_gla_scan.argtypes = [_c_p, _c_i64, _c_int, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p,
                                     _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
         lib.st_gated_head_norm.argtypes = [_c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int,
                                            _c_f, _c_int, _c_p]
         lib.st_latent_write.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
-                                        _c_int, _c_int, _c_f, _c_int, _c_p, _c_int, _c_p]
-        lib.st_moe_route.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_p]
+                                        _c_int, _c_int, _c_f, _c_int, _c_p, _c_f, _c_int, _c_p]
+        lib.st_moe_route.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_moe_align.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_moe_up.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                   _c_f, _c_int, _c_int, _c_p]
@@ -108,6 +108,16 @@ def _lib():
         lib.st_token_side.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
                                       _c_f, _c_int, _c_p]
         lib.st_row_add.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_p]
+        lib.st_scale_softcap.argtypes = [_c_p, _c_i64, _c_f, _c_f, _c_p]
+        lib.st_streams_expand.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_streams_sum.argtypes = [_c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_streams_read.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_streams_write.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_f, _c_int,
+                                         _c_p]
+        lib.st_hashed_embed.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
+                                        _c_int, _c_i64, _c_i64, _c_f, _c_int, _c_int, _c_p]
+        lib.st_qk_norm_write.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int,
+                                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
         _configured = True
@@ -553,14 +563,16 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    num_q_heads: int, scale: float, *, window: int = 0, num_splits: int = 1,
                    num_waves: int = 4, row_ids: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                    workspace: Optional[torch.Tensor] = None, merge: bool = True,
-                   head_slopes: Optional[torch.Tensor] = None):
+                   head_slopes: Optional[torch.Tensor] = None, softcap: float = 0.0):
     """Each query row attends over its request's cached keys [lo, position].
 
     q: [T, num_q_heads*head_dim] view (row stride free).  Returns [T, num_q_heads*head_dim];
     with ``row_ids`` only those batch rows are computed (and written).  ``merge=False`` (with
     num_splits > 1, all rows): the splits are left unmerged and returned as a
     ``SplitAttention`` for a product to merge.  ``head_slopes`` (float32 [num_q_heads]): a head's
-    scaled scores get slope * (key position - query position) added."""
+    scaled scores get slope * (key position - query position) added.  ``window`` > 0: a row reads the last
+    ``window`` positions; < 0: the positions of its own chunk of ``-window`` positions, chunks counted from
+    the sequence's start.  ``softcap`` > 0: scaled scores pass through softcap * tanh(score / softcap)."""
     num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
     T = q.shape[0]
     if head_slopes is not None:
@@ -605,7 +617,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
             o_ptr, _ptr(part_o), _ptr(part_lse), q_ptr, q.stride(0),
             _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), rid_ptr, ti_ptr, po_ptr,
             _ptr(block_table), _ptr(head_slopes), block_table.shape[1], ps, r1 - r0,
-            num_q_heads, nkv, hd, float(scale), int(window), int(num_splits), int(num_waves),
+            num_q_heads, nkv, hd, float(scale), int(window), float(softcap), int(num_splits), int(num_waves),
             dtype_code(q.dtype), _stream()))
     if not merge:
         return SplitAttention(part_o.view(T, num_q_heads, num_splits, hd), part_lse.view(T, num_q_heads, num_splits))
@@ -619,7 +631,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       block_table: torch.Tensor, num_q_heads: int, scale: float, *,
                       window: int = 0, out: Optional[torch.Tensor] = None, key_split: int = 0,
                       tile_rows: int = 64, algo: int = 0,
-                      head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      head_slopes: Optional[torch.Tensor] = None, softcap: float = 0.0) -> torch.Tensor:
     """Tiles of consecutive query rows of prompt portions attend over the cache.
 
     Tile i covers rows [tile_q0[i], tile_q0[i]+tile_rows) of item tile_item[i]; row r of an
@@ -627,8 +639,8 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     ``key_split``: groups of waves that share a tile's key blocks (1, 2 or 4; 0: chosen from
     the number of tiles).  ``tile_rows``: 64, or 128 where ``prefill_tile_rows`` says so.
     ``algo``: 0 chosen by the library, 1 the kernel that stages key blocks through registers,
-    2 the kernel that loads them straight into LDS (it takes no ``head_slopes``, which are as in
-    ``attention_rows``)."""
+    2 the kernel that loads them straight into LDS (it takes no ``head_slopes``, no ``softcap`` and no
+    negative ``window``, which are as in ``attention_rows``)."""
     num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
     T = q.shape[0]
     _need(q, "q", None, (T, num_q_heads * hd), contiguous=False)
@@ -649,7 +661,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0),
         _ptr(tile_item), _ptr(tile_q0), nt, _ptr(item_tok_off), _ptr(item_start), _ptr(item_len),
         _ptr(block_table), _ptr(head_slopes), block_table.shape[1], ps, num_q_heads, nkv, hd, float(scale), int(window),
-        int(key_split), int(tile_rows), int(algo), dtype_code(q.dtype), _stream()))
+        float(softcap), int(key_split), int(tile_rows), int(algo), dtype_code(q.dtype), _stream()))
     return out
 
 
@@ -1054,10 +1066,13 @@ def retention_chunks(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: t
 @_timed("gated_group_norm", lambda o, gate, *a, **k: {"rows": o.shape[0], "width": o.shape[1],
                                                        "bytes": o.numel() * (4 + 3 * gate.element_size())})
 def gated_group_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, groups: int, eps: float,
-                     out_dtype: torch.dtype, gate_first: bool = False) -> torch.Tensor:
+                     out_dtype: torch.dtype, gate_first: bool = False, gate_kind: str = "silu") -> torch.Tensor:
     """Each of the ``groups`` equal parts of a row of o (float [T, W]) divided by its root mean square and
     multiplied by ``gain`` (float [W / groups] shared by the parts, or [W]) and by silu(gate) (``gate``:
-    [T, W] rows of ``out_dtype``, any stride); ``gate_first``: the gate multiplies before the norm."""
+    [T, W] rows of ``out_dtype``, any stride); ``gate_first``: the gate multiplies before the norm;
+    ``gate_kind`` "sigmoid": sigmoid(gate) in silu's place."""
+    if gate_kind not in ("silu", "sigmoid"):
+        raise KernelError(f"the gate is silu or sigmoid, not {gate_kind!r}")
     T, W = o.shape
     if W % groups:
         raise KernelError(f"{W} channels do not divide into {groups} parts")
@@ -1071,7 +1086,8 @@ def gated_group_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, gr
     _need(gain, "gain", torch.float32)
     out = empty((T, W), out_dtype, o.device)
     _check(_lib().st_gated_group_norm(_ptr(out), _ptr(o), _ptr(gate), gate.stride(0), _ptr(gain), T, groups, width,
-                                      int(gain.shape[0] == W and groups > 1), int(bool(gate_first)), float(eps),
+                                      int(gain.shape[0] == W and groups > 1), int(bool(gate_first)),
+                                      int(gate_kind == "sigmoid"), float(eps),
                                       dtype_code(out_dtype), _stream()))
     return out
 
@@ -1168,12 +1184,13 @@ def gated_head_norm(o, gate: torch.Tensor, gain: torch.Tensor, heads: int, eps: 
                                                    "bytes": x.numel() * (4 + cache.element_size())})
 def latent_write(cache: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, token_item: torch.Tensor,
                  positions: torch.Tensor, block_table: torch.Tensor, tail: int = 0,
-                 tail_freq: Optional[torch.Tensor] = None) -> None:
+                 tail_freq: Optional[torch.Tensor] = None, tail_mult: float = 1.0) -> None:
     """Each row of x (float [T, rank + tail], dense rows of any stride): its first ``rank`` values are
     normalised to unit root mean square, multiplied by ``gain`` and stored as its token's entry of ``cache``
     [pages, 1, page_size, entry] with entry >= rank + tail; the ``tail`` values after them follow in the
     entry as they are, or, with ``tail_freq`` (float [tail / 2]), turned by the token's position (pairs
-    2i, 2i + 1; angle position * tail_freq[i]); the rest of an entry is cleared."""
+    2i, 2i + 1; angle position * tail_freq[i]; cosine and sine times ``tail_mult``); the rest of an entry is
+    cleared."""
     num_pages, one, ps, entry = cache.shape
     T = x.shape[0]
     rank = x.shape[1] - int(tail)
@@ -1193,7 +1210,8 @@ def latent_write(cache: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: 
     _need(block_table, "block_table", torch.int32)
     _check(_lib().st_latent_write(_ptr(cache), cache.stride(0), _ptr(x), x.stride(0), _ptr(gain), _ptr(token_item),
                                   _ptr(positions), _ptr(block_table), block_table.shape[1], ps, T, rank, entry,
-                                  float(eps), int(tail), _ptr(tail_freq), dtype_code(cache.dtype), _stream()))
+                                  float(eps), int(tail), _ptr(tail_freq), float(tail_mult), dtype_code(cache.dtype),
+                                  _stream()))
 
 
 # ---------------------------------------------------------------- routed experts
@@ -1222,7 +1240,7 @@ def _d_moe(x, logits, w_gate, w_up, w_down, residual, *, top, limit=0.0, out_sca
 def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
                    w_down: torch.Tensor, residual: Optional[torch.Tensor], *, top: int, limit: float = 0.0,
                    out_scale: float = 1.0, token_item: Optional[torch.Tensor] = None,
-                   style: str = "scaled_input") -> torch.Tensor:
+                   style: str = "scaled_input", groups: int = 1, keep: int = 1) -> torch.Tensor:
     """residual <- residual + out_scale * sum over a row's ``top`` best experts e (by ``logits``) of
     Wd[e] y with y = g * sigmoid(1.702 g) * (u + 1), g = min(s * Wg[e] x, limit),
     u = clamp(s * Wu[e] x, -limit, limit), s = sigmoid(logit of e).  In place on ``residual``
@@ -1231,6 +1249,9 @@ def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, 
     ``style`` "softmax_output": the weights of a row's experts are the softmax over their logits alone and
     multiply the experts' results, sum_e s_e Wd[e] (silu(Wg[e] x) * (Wu[e] x)), with no limit.  Then
     ``residual`` may be None: the weighted sum itself is returned (a new float tensor).
+    ``style`` "softmax_all": the same experts, weighted by their shares of the softmax over all experts' logits
+    (not renormalised); only experts of the ``keep`` best of ``groups`` equal groups of neighbours can be chosen,
+    a group ranking by its largest logit.
 
     x: [T, width]; logits: float [T, experts]; w_gate, w_up: [experts, inner, width]; w_down:
     [experts, width, inner].  Rows whose ``token_item`` is negative are left as they are."""
@@ -1241,9 +1262,12 @@ def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, 
     _need(w_gate, "w_gate", None, (E, F, W))
     _need(w_up, "w_up", w_gate.dtype, (E, F, W))
     _need(w_down, "w_down", w_gate.dtype, (E, W, F))
-    if style not in ("scaled_input", "softmax_output"):
+    if style not in ("scaled_input", "softmax_output", "softmax_all"):
         raise KernelError(f"routed_experts: unknown style {style!r}")
-    on_output = style == "softmax_output"
+    on_output = style != "scaled_input"
+    mode = {"scaled_input": 0, "softmax_output": 1, "softmax_all": 2}[style]
+    if mode == 2 and (groups < 1 or E % groups or not 1 <= keep <= groups or top > keep * (E // groups)):
+        raise KernelError(f"routed_experts: {top} of {E} experts in {groups} groups of which {keep} are kept")
     if residual is None and not on_output:
         raise KernelError("routed_experts: this style adds to a residual stream")
     if residual is not None:
@@ -1259,7 +1283,7 @@ def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, 
     place = empty((T * top,), torch.int32, dev)
     tile_expert = empty((cap // tile,), torch.int32, dev)
     y = empty((cap, F), x.dtype, dev)
-    _check(lib.st_moe_route(_ptr(ids), _ptr(wts), _ptr(logits), _ptr(token_item), T, E, int(top), int(on_output), st))
+    _check(lib.st_moe_route(_ptr(ids), _ptr(wts), _ptr(logits), _ptr(token_item), T, E, int(top), mode, int(groups), int(keep), st))
     _check(lib.st_moe_align(_ptr(sorted_pairs), _ptr(place), _ptr(tile_expert), _ptr(ids), T * top, E, cap, tile, st))
     _check(lib.st_moe_up(_ptr(y), _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(sorted_pairs), _ptr(tile_expert),
                          _ptr(wts), cap, tile, int(top), W, F, float(limit), int(on_output), code, st))
@@ -1383,6 +1407,147 @@ def row_add(x: torch.Tensor, first: Optional[torch.Tensor], vec: torch.Tensor) -
     _need(vec, "vec", torch.float32, (W,))
     out = empty((T, W), torch.float32, x.device)
     _check(_lib().st_row_add(_ptr(out), _ptr(x), _ptr(first), _ptr(vec), T, W, _stream()))
+    return out
+
+
+def scale_softcap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+    """x <- cap * tanh(x * scale / cap) (``cap`` <= 0: x * scale), in place on a dense float tensor."""
+    _need(x, "x", torch.float32)
+    _check(_lib().st_scale_softcap(_ptr(x), x.numel(), float(scale), float(cap), _stream()))
+    return x
+
+
+# ------------------------------------------------ a residual stream of several copies
+def streams_expand(x: torch.Tensor, streams: int) -> torch.Tensor:
+    """[T, W] float -> [T, streams * W]: every stream a copy of the row."""
+    T, W = x.shape
+    _need(x, "x", torch.float32, (T, W))
+    out = empty((T, streams * W), torch.float32, x.device)
+    _check(_lib().st_streams_expand(_ptr(out), _ptr(x), T, int(streams), W, _stream()))
+    return out
+
+
+def streams_sum(x: torch.Tensor, streams: int, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The sum of the streams of x (float [T, streams * W]) for every row, or for the rows picked by ``rows``
+    (int32; a negative entry gives zeros): float [rows, W]."""
+    T, SW = x.shape
+    if SW % streams:
+        raise KernelError(f"{SW} columns are not {streams} streams")
+    W = SW // streams
+    _need(x, "x", torch.float32, (T, SW))
+    n = T
+    if rows is not None:
+        n = rows.shape[0]
+        _need(rows, "rows", torch.int32, (n,))
+    out = empty((n, W), torch.float32, x.device)
+    _check(_lib().st_streams_sum(_ptr(out), _ptr(x), _ptr(rows), n, int(streams), W, _stream()))
+    return out
+
+
+@_timed("streams_read", lambda x, weights, *a, **k: {"rows": x.shape[0], "width": x.shape[1],
+                                                     "bytes": x.numel() * 4 + x.numel() // weights.shape[0] * 2})
+def streams_read(x: torch.Tensor, weights: torch.Tensor, gain: Optional[torch.Tensor], eps: float,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    """u = sum_s weights[s] x_s of the streams x (float [T, S * W]), then u * rsqrt(mean(u^2) + eps) * gain
+    (``eps`` <= 0: u itself) in ``out_dtype``: what a sublayer reads."""
+    T, SW = x.shape
+    S = weights.shape[0]
+    W = SW // S
+    _need(x, "x", torch.float32, (T, S * W))
+    _need(weights, "weights", torch.float32, (S,))
+    if gain is not None:
+        _need(gain, "gain", torch.float32, (W,))
+    out = empty((T, W), out_dtype, x.device)
+    _check(_lib().st_streams_read(_ptr(out), None, _ptr(x), _ptr(weights), _ptr(gain), T, S, W, float(eps),
+                                  dtype_code(out_dtype), _stream()))
+    return out
+
+
+@_timed("streams_write", lambda x, y, mix, *a, **k: {"rows": x.shape[0], "width": x.shape[1],
+                                                     "bytes": x.numel() * 8 + y.numel() * 4})
+def streams_write(x: torch.Tensor, y: torch.Tensor, mix: torch.Tensor, out_weights: torch.Tensor,
+                  then: Optional[tuple] = None, out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """In place on the streams x (float [T, S * W]): x_t <- sum_s mix[s, t] x_s + out_weights[t] * y, y float
+    [T, W].  ``then`` = (weights, gain or None, eps): also returns the next sublayer's read of the new streams
+    (as ``streams_read``) in ``out_dtype``, made in the same pass."""
+    T, SW = x.shape
+    S = out_weights.shape[0]
+    W = SW // S
+    _need(x, "x", torch.float32, (T, S * W))
+    _need(y, "y", torch.float32, (T, W))
+    _need(mix, "mix", torch.float32, (S, S))
+    _need(out_weights, "out_weights", torch.float32, (S,))
+    nxt = a2 = g2 = None
+    eps2, code = 0.0, F32
+    if then is not None:
+        a2, g2, eps2 = then
+        _need(a2, "next weights", torch.float32, (S,))
+        if g2 is not None:
+            _need(g2, "next gain", torch.float32, (W,))
+        nxt = empty((T, W), out_dtype, x.device)
+        code = dtype_code(out_dtype)
+    _check(_lib().st_streams_write(_ptr(x), _ptr(y), _ptr(mix), _ptr(out_weights), _ptr(nxt), _ptr(a2), _ptr(g2), T, S,
+                                   W, float(eps2), code, _stream()))
+    return nxt
+
+
+def hashed_embed(ids: torch.Tensor, positions: torch.Tensor, ctx_arrays, last_token: Optional[torch.Tensor],
+                 table: torch.Tensor, pairs: Optional[torch.Tensor], mul_prev: int, mul_cur: int,
+                 scale: float) -> torch.Tensor:
+    """x[t] = table[id_t] * scale + pairs[(id_(t-1) * mul_prev + id_t * mul_cur) mod buckets], float [T, W];
+    pairs [buckets + 1, W], its last row for a sequence's first token.  ``ctx_arrays`` = (token_item, item_len,
+    item_tok_off, item_slot); ``last_token`` (int32 [slots]): the last token of each slot's request so far,
+    read for an item's first row and moved on to the item's last token of this step.  ``pairs`` None: the
+    token's row times the factor alone."""
+    token_item, item_len, item_tok_off, item_slot = ctx_arrays
+    T = ids.shape[0]
+    V, W = table.shape
+    _need(table, "table", None, (V, W))
+    buckets = 0
+    if pairs is not None:
+        _need(pairs, "pairs", table.dtype, (pairs.shape[0], W))
+        if pairs.shape[0] < 2:
+            raise KernelError("the table of pairs has a row a bucket and one more")
+        buckets = pairs.shape[0] - 1
+        _need(last_token, "last_token", torch.int32)
+    for name, v in (("ids", ids), ("positions", positions), ("token_item", token_item)):
+        _need(v, name, torch.int32, (T,))
+    B = item_len.shape[0]
+    for name, v in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
+        _need(v, name, torch.int32, (B,))
+    out = empty((T, W), torch.float32, table.device)
+    _check(_lib().st_hashed_embed(_ptr(out), _ptr(ids), _ptr(positions), _ptr(token_item), _ptr(item_len),
+                                  _ptr(item_tok_off), _ptr(item_slot), _ptr(last_token), _ptr(table), _ptr(pairs), T, B,
+                                  V, buckets, int(mul_prev), int(mul_cur), float(scale), W,
+                                  dtype_code(table.dtype), _stream()))
+    return out
+
+
+def qk_norm_write(qk: torch.Tensor, gain_q: torch.Tensor, gain_k: torch.Tensor, eps: float, heads: int, kv_heads: int,
+                  head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor, token_item: torch.Tensor,
+                  positions: torch.Tensor, block_table: torch.Tensor, write: bool = True) -> torch.Tensor:
+    """qk: float [T, (heads + kv_heads) * head_dim], queries then keys.  Both are divided by their root mean
+    square over the whole projection and multiplied by their gains; returns the queries [T, heads * head_pad]
+    in the pools' type (head_pad: the pools' entry width, zeros behind head_dim) and, with ``write``, stores
+    the normalised keys in ``k_cache`` and the keys as projected in ``v_cache``."""
+    num_pages, nkv, ps, pad = k_cache.shape
+    T = qk.shape[0]
+    _need(qk, "qk", torch.float32, (T, (heads + kv_heads) * head_dim), contiguous=False)
+    if qk.stride(1) != 1:
+        raise KernelError("qk: rows must be dense")
+    if nkv != kv_heads or pad < head_dim or tuple(v_cache.shape) != tuple(k_cache.shape) or \
+            k_cache.stride()[1:] != (ps * pad, pad, 1) or v_cache.stride() != k_cache.stride():
+        raise KernelError("qk_norm_write: the pools do not fit the keys")
+    _need(gain_q, "gain_q", torch.float32, (heads * head_dim,))
+    _need(gain_k, "gain_k", torch.float32, (kv_heads * head_dim,))
+    _need(token_item, "token_item", torch.int32, (T,))
+    _need(positions, "positions", torch.int32, (T,))
+    _need(block_table, "block_table", torch.int32)
+    out = empty((T, heads * pad), k_cache.dtype, qk.device)
+    _check(_lib().st_qk_norm_write(_ptr(out), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), _ptr(qk), qk.stride(0),
+                                   _ptr(gain_q), _ptr(gain_k), _ptr(token_item), _ptr(positions), _ptr(block_table),
+                                   block_table.shape[1], ps, T, heads, kv_heads, head_dim, pad, float(eps), int(write),
+                                   dtype_code(k_cache.dtype), _stream()))
     return out
 
 

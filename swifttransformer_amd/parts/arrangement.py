@@ -9,12 +9,18 @@ post-norm (the reference refuses it, gpt.cc:238-240):
 sandwich (norms before and after each sublayer; the reference has no such block):
     r = x + N1b(Mix(N1(x))); s = r + N2b(FFN(N2(r))); x' = s + Side(s, token)
     (the feed-forward and the side input are optional)
+hyper-connections (several copies of the stream; the reference has no such block):
+    u = sum_s a1[s] x_s;  y = Mix(N1(u));  x_t <- sum_s M1[s, t] x_s + b1[t] y   (all t at once)
+    and the same with a2, M2, b2 around the feed-forward, which is optional
 The residual stream is float; parts that multiply matrices take the storage type."""
 from __future__ import annotations
 
 import torch
 
+from typing import Dict, List
+
 from ..ops import kernels as K
+from ..weights.loader import TensorSpec
 from .base import Part
 
 
@@ -110,3 +116,76 @@ def _chains(norm, then) -> bool:
     """Whether ``norm.forward_onto`` can make a second result in the same pass (``then``: another norm of its
     kind, or None for the plain sum in the storage type)."""
     return getattr(norm, "chains_onto", False) and (then is None or type(then) is type(norm))
+
+
+class HyperConnections(Part):
+    """params: streams (int), feed_forward (bool, default True).  names: ``mixer_in``, ``mixer_out`` (float
+    [streams]), ``mixer_mix`` ([streams, streams], indexed [from, to]) and ``ffn_in``, ``ffn_out``, ``ffn_mix``.
+
+    The stream it is handed is float [T, streams * hidden]: the model makes the copies after the embedding
+    and sums them before the final norm (``ModelSpec.streams``).  It is updated in place.  The sublayers are
+    asked for their results alone (``raw_output_ok``).  Where a norm is the root-mean-square form with a gain,
+    the weighted sum of the streams and the norm are one kernel, and the write after the mixer makes the
+    feed-forward's input in the same pass."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        super().__init__(spec, hidden_size, dtype)
+        self.streams = int(self.param("streams"))
+        if not 1 <= self.streams <= 16:
+            raise ValueError(f"1 to 16 streams, not {self.streams}")
+        self.has_ffn = bool(spec.params.get("feed_forward", True))
+        self.needs = ("mixer_norm", "ffn_norm", "feed_forward") if self.has_ffn else ("mixer_norm",)
+        self.w = {}
+
+    def _sides(self):
+        return ("mixer", "ffn") if self.has_ffn else ("mixer",)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        S = self.streams
+        specs = []
+        for side in self._sides():
+            specs += [TensorSpec(self.name(side + "_in"), (S,), "vector", init="gain"),
+                      TensorSpec(self.name(side + "_out"), (S,), "vector", init="gain"),
+                      TensorSpec(self.name(side + "_mix"), (S, S), "vector", init="mix")]
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for side in self._sides():
+            for what in ("in", "out", "mix"):
+                self.w[side, what] = tensors[self.name(f"{side}_{what}")].contiguous()
+
+    @staticmethod
+    def _plain_rms(norm):
+        """(gain, eps) of a norm that the stream kernels can apply themselves, else None."""
+        if (type(norm).__name__ == "LayerNorm" and not norm.center and norm.beta is None and norm.affine):
+            return norm.gamma, norm.eps
+        return None
+
+    def _read(self, x32, side: str, norm):
+        fused = self._plain_rms(norm)
+        if fused is not None:
+            return K.streams_read(x32, self.w[side, "in"], fused[0], fused[1], self.dtype)
+        u32 = K.streams_read(x32, self.w[side, "in"], None, 0.0, torch.float32)
+        return norm.forward(u32, out_t=True)[0]
+
+    def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True) -> torch.Tensor:
+        for part in (layer.mixer, layer.feed_forward if self.has_ffn else None):
+            if part is not None and not getattr(part, "raw_output_ok", False):
+                raise ValueError(f"{type(part).__name__} cannot give its result without the residual stream")
+        if x32.shape[1] != self.streams * self.hidden_size:
+            raise ValueError(f"{self.streams} streams of {self.hidden_size} make no row of {x32.shape[1]}")
+        a = self._read(x32, "mixer", layer.mixer_norm)
+        m32 = layer.mixer.forward(a, None, ctx, cache, write)
+        if not self.has_ffn:
+            K.streams_write(x32, m32, self.w["mixer", "mix"], self.w["mixer", "out"])
+            return x32
+        fused = self._plain_rms(layer.ffn_norm)
+        if fused is not None:
+            d = K.streams_write(x32, m32, self.w["mixer", "mix"], self.w["mixer", "out"],
+                                then=(self.w["ffn", "in"], fused[0], fused[1]), out_dtype=self.dtype)
+        else:
+            K.streams_write(x32, m32, self.w["mixer", "mix"], self.w["mixer", "out"])
+            d = self._read(x32, "ffn", layer.ffn_norm)
+        f32 = layer.feed_forward.forward(d, None, ctx)
+        K.streams_write(x32, f32, self.w["ffn", "mix"], self.w["ffn", "out"])
+        return x32

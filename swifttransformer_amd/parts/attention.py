@@ -155,13 +155,17 @@ class PagedAttention(Mixer):
         return self.plan_key(), planner
 
     # ------------------------------------------------------------------ forward
+    def key_span(self, ctx) -> int:
+        """The most keys a row of this step reads."""
+        return ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
+
     def _shape_row_kernel(self, ctx, rows: int):
         """(key splits, waves per workgroup) of the row kernel.  A workgroup serves one
         (row, head, split); when rows * heads alone does not fill the chip, a row's keys are
         split over workgroups (merged by a second kernel), at least tuning.min_keys_per_split keys
         each.  ctx.max_kv_len is the longest sequence of this step, or, for a recorded step,
         the longest the model allows: then the shape depends on the batch size alone."""
-        span = ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
+        span = self.key_span(ctx)
         groups = max(1, rows * self.num_heads)
         units = _target_workgroups()
         splits = min(-(-units // groups), max(1, span // tuning.min_keys_per_split), 32)

@@ -43,3 +43,12 @@ register_part("mixer", "gated_window_attention", GatedWindowAttention)
 register_part("mixer", "retention", Retention)
 register_part("mixer", "parallel", ParallelMixers)
 register_part("side_input", "token_side", TokenSideInput)
+from .arrangement import HyperConnections
+from .embedding import HashedPairEmbedding
+from .feed_forward import GatedFeedForward
+from .tied_attention import TiedKeyValueAttention
+
+register_part("arrangement", "hyper_connections", HyperConnections)
+register_part("embedding", "hashed_pairs", HashedPairEmbedding)
+register_part("feed_forward", "gated_dense", GatedFeedForward)
+register_part("mixer", "tied_kv_attention", TiedKeyValueAttention)

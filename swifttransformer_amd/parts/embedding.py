@@ -6,7 +6,10 @@ projected first (no bias) and the position rows are added to the projected
 vector; the reference has no such model (README.md:42 tells users to avoid it).
 The head computes logits = y * Wlm^T in float (src/csrc/model/gpt/gpt.cc:192-201),
 after an optional output projection, and falls back to the embedding table when
-the file has no separate head tensor (tied weights, scripts/lib/converter_lib.py:272)."""
+the file has no separate head tensor (tied weights, scripts/lib/converter_lib.py:272).
+``HashedPairEmbedding`` adds a row of a second table chosen by a hash of the token and the token before it
+in its sequence, and multiplies the token's own row by a factor; the head may multiply its logits by a factor
+and limit them smoothly, cap * tanh(logit / cap).  The reference has neither."""
 from __future__ import annotations
 
 from typing import Dict, List, Optional
@@ -78,9 +81,51 @@ class TokenEmbedding(Part):
         return x32
 
 
+class HashedPairEmbedding(Part):
+    """params: vocab_size, scale (float, default 1: the factor on the token's row), buckets, mul_prev, mul_cur
+    (ints: the row of ``pairs`` is (previous token * mul_prev + token * mul_cur) mod buckets; a sequence's first
+    token takes row ``buckets``, the last one; buckets 0: no second table).  names: weight [vocab, hidden], pairs [buckets + 1, hidden].
+
+    The previous token of a step's first row is the request's last token of an earlier step: one int a
+    request in its state slot (``cache_need``), which the model hands to ``forward`` as ``cache``."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        super().__init__(spec, hidden_size, dtype)
+        self.vocab_size = int(self.param("vocab_size"))
+        self.scale = float(spec.params.get("scale", 1.0))
+        self.buckets = int(self.param("buckets"))
+        self.mul_prev = int(spec.params.get("mul_prev", 1))
+        self.mul_cur = int(spec.params.get("mul_cur", 1))
+        if self.buckets < 0:
+            raise ValueError(f"the number of buckets is not negative ({self.buckets}); 0: no table of pairs")
+        self.table = self.pairs = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [TensorSpec(self.name("weight"), (self.vocab_size, self.hidden_size), "table")]
+        if self.buckets:
+            specs.append(TensorSpec(self.name("pairs"), (self.buckets + 1, self.hidden_size), "table"))
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.table = tensors[self.name("weight")]
+        self.pairs = tensors[self.name("pairs")] if self.buckets else None
+
+    def cache_need(self):
+        from .base import CacheNeed
+        return CacheNeed("state", state_shape=(1,), state_dtype=torch.int32) if self.buckets else None
+
+    def forward(self, ctx, position, cache=None) -> torch.Tensor:
+        if self.buckets and (cache is None or cache.state is None):
+            raise ValueError("the pair embedding keeps each request's last token in its state slot")
+        return K.hashed_embed(ctx.token_ids, ctx.positions, (ctx.token_item, ctx.item_len, ctx.item_tok_off, ctx.item_slot),
+                              cache.state if self.buckets else None, self.table, self.pairs, self.mul_prev,
+                              self.mul_cur, self.scale)
+
+
 class LMHead(Part):
     """params: vocab_size, embed_dim (input width of the head matrix), tied_to (file name of
-    the tensor used when the head's own tensor is absent, or None)."""
+    the tensor used when the head's own tensor is absent, or None), logit_scale (float, default 1) and
+    softcap (float, default 0 = none): logits leave as softcap * tanh(logit_scale * logit / softcap)."""
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
@@ -88,6 +133,8 @@ class LMHead(Part):
         self.embed_dim = int(self.param("embed_dim", hidden_size))
         self.projected = self.embed_dim != hidden_size
         self.tied_to: Optional[str] = spec.params.get("tied_to")
+        self.logit_scale = float(spec.params.get("logit_scale", 1.0))
+        self.softcap = float(spec.params.get("softcap", 0.0) or 0.0)
         self.weight = None
         self.w_out = None
 
@@ -112,7 +159,8 @@ class LMHead(Part):
         """Whether ``forward`` can take ``norm`` (a norm part) of picked rows as its input instead of
         normalised rows, and report the rows' best outputs: the product with the head matrix then
         runs in the kernel that walks a very wide matrix with few rows."""
-        return (not self.projected and hasattr(norm, "as_input") and getattr(norm, "width", None) == self.embed_dim
+        # (the rows' best outputs are found before the factor and the limit: both must keep their order)
+        return (self.logit_scale > 0 and not self.projected and hasattr(norm, "as_input") and getattr(norm, "width", None) == self.embed_dim
                 and K.wide_offered(rows, self.vocab_size, self.embed_dim, self.dtype))
 
     def forward(self, y_t, best: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -121,4 +169,7 @@ class LMHead(Part):
         row's best output, the lowest index on ties."""
         if self.projected:
             y_t = K.gemm(y_t, self.w_out)
-        return K.gemm(y_t, self.weight, out_f32=True, best=best)
+        logits = K.gemm(y_t, self.weight, out_f32=True, best=best)
+        if self.logit_scale != 1.0 or self.softcap > 0:
+            K.scale_softcap(logits, self.logit_scale, self.softcap)
+        return logits

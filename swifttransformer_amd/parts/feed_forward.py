@@ -59,3 +59,37 @@ class DenseFeedForward(Part):
         x_in = norm.as_input(residual32) if norm is not None else x_t
         h = K.gemm(x_in, self.w1, bias=self.b1, activation=self.activation)
         return K.gemm(h, self.w2, bias=self.b2, residual=residual32, out_f32=True, out_scale=self.residual_scale)
+
+
+class GatedFeedForward(Part):
+    """y = Wd (act(Wg x) * (Wu x)), no biases.  params: inner (int), activation (a name the elementwise kernels
+    know), residual_scale (float, default 1).  names: gate, up [inner, hidden], down [hidden, inner].
+    Gate and up are one product; ``forward(..., residual32=None)`` returns the float result alone.
+    The reference has no gated feed-forward."""
+
+    raw_output_ok = True
+
+    def __init__(self, spec, hidden_size, dtype):
+        super().__init__(spec, hidden_size, dtype)
+        self.inner = int(self.param("inner"))
+        self.activation = str(self.param("activation", "silu"))
+        if self.activation not in K.ACTIVATIONS:
+            raise ValueError(f"feed-forward activation {self.activation!r} has no kernel; "
+                             f"available: {sorted(K.ACTIVATIONS)}")
+        self.residual_scale = float(spec.params.get("residual_scale", 1.0))
+        self.w_gate_up = self.w_down = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        H, F = self.hidden_size, self.inner
+        return [TensorSpec(self.name("gate"), (F, H), "matrix"), TensorSpec(self.name("up"), (F, H), "matrix"),
+                TensorSpec(self.name("down"), (H, F), "matrix")]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.w_gate_up = torch.cat([tensors[self.name("gate")], tensors[self.name("up")]], dim=0).contiguous()
+        self.w_down = tensors[self.name("down")]
+
+    def forward(self, x_t, residual32, ctx, norm=None):
+        F = self.inner
+        gu = K.gemm(x_t, self.w_gate_up)
+        h = K.activation_multiply(gu[:, :F], gu[:, F:], self.activation)
+        return K.gemm(h, self.w_down, residual=residual32, out_f32=True, out_scale=self.residual_scale)

@@ -65,13 +65,13 @@ class LatentAttention(PagedAttention):
         if self.rot_dim and not self.own_latent:
             raise ValueError("a latent attention with a turned key part caches it with its own latent")
         self._freq_host = self.freq = None
+        self.rot_mult = 1.0
         if self.rot_dim:
             dims = int(p.get("rot_dims", self.rot_dim) or self.rot_dim)
             if dims % 2 or not 0 < dims <= self.rot_dim:
                 raise ValueError(f"{dims} turning coordinates in a part of {self.rot_dim}")
-            freq, mult = rotary_frequencies(dims, float(p["rot_base"]), p.get("rot_scaling"))
-            if mult != 1.0:
-                raise ValueError("this rule of rescaled frequencies also scales cosine and sine; not offered here")
+            # (a rule that also scales cosine and sine scales the turned parts of queries and keys alike)
+            freq, self.rot_mult = rotary_frequencies(dims, float(p["rot_base"]), p.get("rot_scaling"))
             freq = list(freq) + [0.0] * ((self.rot_dim - dims) // 2)      # an angle of zero leaves a pair as it is
             self._freq_host = torch.tensor(freq, dtype=torch.float64).to(torch.float32)
 
@@ -121,9 +121,9 @@ class LatentAttention(PagedAttention):
         if write:
             raw = K.gemm(x_t, self.w_down, out_f32=True)
             K.latent_write(cache.k, raw, self.gain, self.eps, ctx.token_item, ctx.positions,
-                           ctx.block_tables[cache.group], tail=self.rot_dim, tail_freq=self.freq)
+                           ctx.block_tables[cache.group], tail=self.rot_dim, tail_freq=self.freq, tail_mult=self.rot_mult)
         q = K.gemm(x_t, self.w_q)
         if self.rot_dim:
-            K.rotary(q, None, self.entry, self.freq, 1.0, ctx.positions, offset=self.rank, interleaved=True)
+            K.rotary(q, None, self.entry, self.freq, self.rot_mult, ctx.positions, offset=self.rank, interleaved=True)
         o = self.attend(q, ctx, cache, unmerged_ok=True)
         return K.gemm(o, self.w_out, residual=residual32, out_f32=True, out_scale=self.residual_scale)

@@ -56,6 +56,10 @@ class ModelSpec:
     # parts of the category "reentry": what happens to the residual stream before the runs that name
     # them (a pass over a group of layers that starts from a mix of the stream and the embedding)
     entries: List[PartSpec] = field(default_factory=list)
+    # > 0: the residual stream runs as that many copies side by side, float [T, streams * hidden]: the model
+    # makes the copies after the embedding and sums them before the final norm; the layers' arrangements read
+    # and write all of them
+    streams: int = 0
 
     def validate(self) -> "ModelSpec":
         n = len(self.layers)
