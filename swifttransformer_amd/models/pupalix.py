@@ -61,9 +61,11 @@ def build_pupalix_spec(hp: PupalixHyperParam) -> ModelSpec:
         p = f"l{i}"
         ffn = _feed_forward(f"{p}.mlp", L.get("mlp"))
         if hp.streams:
-            arrangement = PartSpec("hyper_connections", {"streams": hp.streams, "feed_forward": ffn is not None},
-                                   {f"{side}_{what}": f"{p}.{hc}.{what}" for side, hc in (("mixer", "hc1"), ("ffn", "hc2"))
-                                    for what in ("in", "out", "mix")})
+            names = {f"{side}_{what}": f"{p}.{hc}.{what}" for side, hc in (("mixer", "hc1"), ("ffn", "hc2"))
+                     for what in ("in", "out", "mix")}
+            if ffn is None:
+                names["unused_norm"] = f"{p}.norm2"
+            arrangement = PartSpec("hyper_connections", {"streams": hp.streams, "feed_forward": ffn is not None}, names)
         else:
             arrangement = PartSpec("pre_norm", {"feed_forward": ffn is not None})
         layers.append(LayerSpec(

@@ -147,6 +147,11 @@ class HyperConnections(Part):
             specs += [TensorSpec(self.name(side + "_in"), (S,), "vector", init="gain"),
                       TensorSpec(self.name(side + "_out"), (S,), "vector", init="gain"),
                       TensorSpec(self.name(side + "_mix"), (S, S), "vector", init="mix")]
+        if not self.has_ffn:
+            # a layer without feed-forward: a file may still hold the second sublayer's weights; they are not read
+            for what, shape in (("ffn_in", (S,)), ("ffn_out", (S,)), ("ffn_mix", (S, S)), ("unused_norm", (self.hidden_size,))):
+                if what in self.spec.names:
+                    specs.append(TensorSpec(self.name(what), shape, "vector", optional=True))
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:

@@ -228,3 +228,51 @@ class PlainPupalix:
             after.append(x.clone())
         logits = head(x, t["embed"], t["final.norm"], eps, cfg.get("logit_scale", 1.0), cfg.get("logit_softcap"))
         return (logits, torch.stack(after)) if layers else logits
+
+
+def load_folder(folder: str):
+    """(config, float64 tensors by name) of a model folder, through this file's own reader."""
+    import json
+    import os
+    import struct
+    import numpy as np
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    with open(os.path.join(folder, "model.safetensors"), "rb") as f:
+        n = struct.unpack("<Q", f.read(8))[0]
+        meta = json.loads(f.read(n))
+        data = f.read()
+    out = {}
+    for name, m in meta.items():
+        if name == "__metadata__":
+            continue
+        a, b = m["data_offsets"]
+        raw = np.frombuffer(data[a:b], dtype=np.uint8)
+        if m["dtype"] == "BF16":
+            u = raw.view("<u2").astype(np.uint32) << 16
+            t = torch.from_numpy(u.view(np.float32).copy())
+        elif m["dtype"] == "F32":
+            t = torch.from_numpy(raw.view("<f4").copy())
+        else:
+            raise ValueError(m["dtype"])
+        out[name] = t.reshape(m["shape"]).to(F)
+    return cfg, out
+
+
+def logits(cfg, w, tokens):
+    with torch.no_grad():
+        return PlainPupalix(cfg, w).forward(list(tokens))
+
+
+def residual_streams(cfg, w, tokens):
+    with torch.no_grad():
+        return PlainPupalix(cfg, w).forward(list(tokens), layers=True)[1]
+
+
+def generate(cfg, w, prompt, n):
+    seq, out = list(prompt), []
+    for _ in range(n):
+        tok = int(logits(cfg, w, seq)[-1].argmax())
+        out.append(tok)
+        seq.append(tok)
+    return out
