@@ -22,7 +22,8 @@ def _library():
     lib.st_last_error.restype = ctypes.c_char_p
     lib.st_attn_rows_static_capacity.restype = ctypes.c_size_t
     lib.st_attn_rows_static.argtypes = [_p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p] + [_i] * 6 + [_f] + [_i] * 4 + [_p]
-    lib.st_attn_rows.argtypes = [_p, _p, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p] + [_i] * 6 + [_f] + [_i] * 4 + [_p]
+    lib.st_attn_rows.argtypes = ([_p, _p, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p] + [_i] * 6 + [_f, _i, _f] + [_i] * 3 +
+                                 [_p])
     return lib
 
 
@@ -89,9 +90,11 @@ def _run(lib, rows, heads, hd, ctx_len, page, splits, dtype, seed, capture=False
     want = torch.zeros((rows, heads * hd), dtype=dtype, device=DEV)
     work = torch.empty(rows * heads * splits * (hd + 1), dtype=torch.float32, device=DEV)
     n_o = rows * heads * splits * hd
+    t = tail(stream)
+    with_cap = t[:8] + (0.0,) + t[8:]          # this entry point also takes a cap on the scores, after the window
     rc = lib.st_attn_rows(want.data_ptr(), work.data_ptr(), work.data_ptr() + 4 * n_o, q.data_ptr(), q.stride(0),
                           k.data_ptr(), v.data_ptr(), k.stride(0), None, item.data_ptr(), pos.data_ptr(),
-                          table.data_ptr(), None, *tail(stream))
+                          table.data_ptr(), None, *with_cap)
     assert rc == 0, lib.st_last_error().decode()
     _check(want, ref, dtype, "st_attn_rows against dense attention")
     # the entry point under test: the device's free memory does not move across the call
