@@ -209,7 +209,7 @@ def kernel_times(args) -> int:
 
 
 def side_by_side(args, shape: str, other: str = "zitupel", beside=("opt",)) -> int:
-    """Another architecture (Zitupel, Zimorax, Gisedra) beside OPT (``beside``: or other families) at the same layer sizes (width, heads, feed-forward width of OPT
+    """Another architecture (Zitupel, Zimorax, Gisedra, Pupalix) beside OPT (``beside``: or other families) at the same layer sizes (width, heads, feed-forward width of OPT
     ``shape``; the same number of layers, 8 unless ``--layers`` says otherwise; random weights):
     decode tokens/s at batch 1, 8 and 64 from 1,024-token prompts, a 2,048-token prefill, and for
     both the per-kernel times of one decode step at batch ``--batch`` and of the prefill with their
@@ -265,16 +265,26 @@ def side_by_side(args, shape: str, other: str = "zitupel", beside=("opt",)) -> i
                     return seen, seen
                 return keys_read, sum(min(i + 1, w) for i in range(keys_read))
 
+            def chunked(info):
+                # (keys read, query-key pairs) of an attention in chunks of c positions counted from the sequence's
+                # start: a decode row at position p reads p % c + 1 keys, a prompt's row i reads i % c + 1
+                c = -info["window"]
+                if pairs == keys_read:
+                    seen = info["rows"] * ((keys_read // max(info["rows"], 1) - 1) % c + 1)
+                    return seen, seen
+                return keys_read, sum(i % c + 1 for i in range(keys_read))
+
             def nbytes(name, info):
                 if name in ("attention_rows", "attention_prefill"):
-                    return 2 * keys_read * info["kv_heads"] * info["head_dim"] * info["elem"]
+                    keys = chunked(info)[0] if info.get("window", 0) < 0 else keys_read
+                    return 2 * keys * info["kv_heads"] * info["head_dim"] * info["elem"]
                 if name == "sink_attention":
                     return windowed(info)[0] * info["kv_heads"] * (info["head_dim"] + info["value_dim"]) * info["elem"]
                 return None
 
             def flops(name, info):
                 if name in ("attention_rows", "attention_prefill"):
-                    return 4.0 * pairs * info["heads"] * info["head_dim"]
+                    return 4.0 * (chunked(info)[1] if info.get("window", 0) < 0 else pairs) * info["heads"] * info["head_dim"]
                 if name == "sink_attention":
                     return 2.0 * windowed(info)[1] * info["heads"] * (info["head_dim"] + info["value_dim"] + info["heads"])
                 return None
@@ -591,10 +601,12 @@ def main() -> int:
                     choices=["decode-1.3b", "mixed-6.7b", "mixed-1.3b", "ttft", "decode-30b", "decode-family",
                              "zitupel-125m", "zitupel-1.3b", "zitupel-6.7b",
                              "zimorax-125m", "zimorax-1.3b", "zimorax-6.7b",
-                             "gisedra-125m", "gisedra-1.3b", "gisedra-6.7b"],
+                             "gisedra-125m", "gisedra-1.3b", "gisedra-6.7b",
+                             "pupalix-125m", "pupalix-1.3b", "pupalix-6.7b"],
                     help="decode-1.3b is the default line; the others are the other model shapes; zitupel-<size>, "
                          "zimorax-<size>: that architecture beside OPT at the same layer sizes; gisedra-<size>: "
-                         "Gisedra beside Zitupel and Zimorax (whose kernels are its kernels' likes) and OPT")
+                         "Gisedra beside Zitupel and Zimorax (whose kernels are its kernels' likes) and OPT; "
+                         "pupalix-<size>: Pupalix beside Gisedra, Zitupel and OPT")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -622,6 +634,8 @@ def main() -> int:
         return side_by_side(args, shape, family)
     if args.workload.startswith("gisedra-"):
         return side_by_side(args, args.workload.split("-", 1)[1], "gisedra", beside=("zitupel", "zimorax", "opt"))
+    if args.workload.startswith("pupalix-"):
+        return side_by_side(args, args.workload.split("-", 1)[1], "pupalix", beside=("gisedra", "zitupel", "opt"))
     steps = min(args.steps, CONTEXT - PROMPT_LEN)
     elem = 2 if args.dtype == "bf16" else 4
     biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)

@@ -548,13 +548,19 @@ def _d_attention_rows(q, k_cache, v_cache, token_item, positions, block_table, n
                       num_splits=1, row_ids=None, merge=True, **kw):
     # how many keys the rows read is on the device only: the caller of the timer knows its workload
     rows = row_ids.shape[0] if row_ids is not None else q.shape[0]
-    return {"rows": rows, "heads": num_q_heads, "kv_heads": k_cache.shape[1], "head_dim": k_cache.shape[3],
+    info = {"rows": rows, "heads": num_q_heads, "kv_heads": k_cache.shape[1], "head_dim": k_cache.shape[3],
             "splits": num_splits, "merged": bool(merge), "elem": k_cache.element_size()}
+    if kw.get("window"):
+        info["window"] = int(kw["window"])       # negative: chunks of that many positions
+    return info
 
 
 def _d_attention_prefill(q, k_cache, v_cache, tile_item, *a, **kw):
-    return {"rows": q.shape[0], "tiles": tile_item.shape[0], "heads": q.shape[1] // k_cache.shape[3],
+    info = {"rows": q.shape[0], "tiles": tile_item.shape[0], "heads": q.shape[1] // k_cache.shape[3],
             "kv_heads": k_cache.shape[1], "head_dim": k_cache.shape[3], "elem": k_cache.element_size()}
+    if kw.get("window"):
+        info["window"] = int(kw["window"])
+    return info
 
 
 @_timed("attention_rows", _d_attention_rows)
@@ -1410,6 +1416,7 @@ def row_add(x: torch.Tensor, first: Optional[torch.Tensor], vec: torch.Tensor) -
     return out
 
 
+@_timed("scale_softcap", lambda x, *a, **k: {"rows": x.shape[0], "width": x.shape[-1], "bytes": 8 * x.numel()})
 def scale_softcap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
     """x <- cap * tanh(x * scale / cap) (``cap`` <= 0: x * scale), in place on a dense float tensor."""
     _need(x, "x", torch.float32)
@@ -1418,6 +1425,7 @@ def scale_softcap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torc
 
 
 # ------------------------------------------------ a residual stream of several copies
+@_timed("streams_expand", lambda x, streams: {"rows": x.shape[0], "width": x.shape[1], "bytes": 4 * x.numel() * (1 + streams)})
 def streams_expand(x: torch.Tensor, streams: int) -> torch.Tensor:
     """[T, W] float -> [T, streams * W]: every stream a copy of the row."""
     T, W = x.shape
@@ -1491,6 +1499,9 @@ def streams_write(x: torch.Tensor, y: torch.Tensor, mix: torch.Tensor, out_weigh
     return nxt
 
 
+@_timed("hashed_embed", lambda ids, positions, ctx_arrays, last_token, table, pairs, *a, **k: {
+    "rows": ids.shape[0], "width": table.shape[1],
+    "bytes": ids.shape[0] * table.shape[1] * (4 + table.element_size() * (2 if pairs is not None else 1))})
 def hashed_embed(ids: torch.Tensor, positions: torch.Tensor, ctx_arrays, last_token: Optional[torch.Tensor],
                  table: torch.Tensor, pairs: Optional[torch.Tensor], mul_prev: int, mul_cur: int,
                  scale: float) -> torch.Tensor:
@@ -1523,6 +1534,9 @@ def hashed_embed(ids: torch.Tensor, positions: torch.Tensor, ctx_arrays, last_to
     return out
 
 
+@_timed("qk_norm_write", lambda qk, gain_q, gain_k, eps, heads, kv_heads, head_dim, k_cache, *a, **k: {
+    "rows": qk.shape[0], "width": qk.shape[1],
+    "bytes": qk.shape[0] * (4 * qk.shape[1] + k_cache.element_size() * k_cache.shape[3] * (heads + 2 * kv_heads))})
 def qk_norm_write(qk: torch.Tensor, gain_q: torch.Tensor, gain_k: torch.Tensor, eps: float, heads: int, kv_heads: int,
                   head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor, token_item: torch.Tensor,
                   positions: torch.Tensor, block_table: torch.Tensor, write: bool = True) -> torch.Tensor:
