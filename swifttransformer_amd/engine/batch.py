@@ -63,6 +63,9 @@ class StepContext:
     # work lists that parts asked for through their ``step_planner`` (key -> StepPlan); a key is
     # absent when its planner had nothing to say about this batch, and in recorded steps
     plans: Dict[Hashable, "StepPlan"] = field(default_factory=dict)
+    # what one run of a layer has made for the next one on its last pass over the stream (an arrangement that
+    # reads ahead leaves it here and the next run takes it): (tensor, address of the stream it was made from)
+    read_ahead: Optional[tuple] = None
 
 
 # A planner looks at the items of a step on the host (and at the page size and table width) and

@@ -170,6 +170,7 @@ class DecoderModel:
             # the reference refuses to run before weights are loaded (gptop_base.cc:47-49)
             raise RuntimeError("load the weights before running the model")
         ctx.position = self.position
+        ctx.read_ahead = None
         embed = ((lambda: self.embedding.forward(ctx, self.position, cache=caches.get(EMBEDDING_CACHE)))
                  if hasattr(self.embedding, "cache_need") else (lambda: self.embedding.forward(ctx, self.position)))
         if self.entries:
@@ -192,6 +193,12 @@ class DecoderModel:
             if layer.mixer_conv is not None:
                 x32 = layer.arrangement.forward(x32, layer, ctx, cache, e.write,
                                                 conv_cache=caches.get(conv_cache_id(run)))
+            elif getattr(layer.arrangement, "reads_ahead", False):
+                # an arrangement whose last pass over the stream can make the next run's first input on the way:
+                # it is told which layer follows (none before a run that is entered through a part of its own)
+                nxt = self.schedule[run + 1] if run + 1 < len(self.schedule) else None
+                follows = self.layers[nxt.layer] if nxt is not None and nxt.enter is None else None
+                x32 = layer.arrangement.forward(x32, layer, ctx, cache, e.write, then=follows)
             else:
                 x32 = layer.arrangement.forward(x32, layer, ctx, cache, e.write)
         return x32

@@ -126,7 +126,11 @@ class HyperConnections(Part):
     and sums them before the final norm (``ModelSpec.streams``).  It is updated in place.  The sublayers are
     asked for their results alone (``raw_output_ok``).  Where a norm is the root-mean-square form with a gain,
     the weighted sum of the streams and the norm are one kernel, and the write after the mixer makes the
-    feed-forward's input in the same pass."""
+    feed-forward's input in the same pass.  ``forward(..., then=layer)``: the layer that runs next; where it
+    is of this kind, the layer's last write also makes that layer's mixer input (``reads_ahead``) and leaves
+    it with the step's context, where the next run finds it."""
+
+    reads_ahead = True
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
@@ -173,16 +177,33 @@ class HyperConnections(Part):
         u32 = K.streams_read(x32, self.w[side, "in"], None, 0.0, torch.float32)
         return norm.forward(u32, out_t=True)[0]
 
-    def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True) -> torch.Tensor:
+    def _ahead(self, then):
+        """What the last write of this layer can make for the layer ``then``: (weights, gain, eps), or None."""
+        if then is None or type(then.arrangement) is not type(self) or then.arrangement.streams != self.streams:
+            return None
+        fused = self._plain_rms(then.mixer_norm)
+        return None if fused is None else (then.arrangement.w["mixer", "in"], fused[0], fused[1])
+
+    def _last_write(self, x32, y32, side: str, then, ctx) -> None:
+        ahead = self._ahead(then)
+        made = K.streams_write(x32, y32, self.w[side, "mix"], self.w[side, "out"], then=ahead,
+                               out_dtype=self.dtype if ahead is not None else None)
+        ctx.read_ahead = (made, x32.data_ptr()) if ahead is not None else None
+
+    def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True, then=None) -> torch.Tensor:
         for part in (layer.mixer, layer.feed_forward if self.has_ffn else None):
             if part is not None and not getattr(part, "raw_output_ok", False):
                 raise ValueError(f"{type(part).__name__} cannot give its result without the residual stream")
         if x32.shape[1] != self.streams * self.hidden_size:
             raise ValueError(f"{self.streams} streams of {self.hidden_size} make no row of {x32.shape[1]}")
-        a = self._read(x32, "mixer", layer.mixer_norm)
+        ahead, ctx.read_ahead = getattr(ctx, "read_ahead", None), None
+        if ahead is not None and ahead[1] == x32.data_ptr():
+            a = ahead[0]                     # the run before this one has made it with its last write
+        else:
+            a = self._read(x32, "mixer", layer.mixer_norm)
         m32 = layer.mixer.forward(a, None, ctx, cache, write)
         if not self.has_ffn:
-            K.streams_write(x32, m32, self.w["mixer", "mix"], self.w["mixer", "out"])
+            self._last_write(x32, m32, "mixer", then, ctx)
             return x32
         fused = self._plain_rms(layer.ffn_norm)
         if fused is not None:
@@ -192,5 +213,5 @@ class HyperConnections(Part):
             K.streams_write(x32, m32, self.w["mixer", "mix"], self.w["mixer", "out"])
             d = self._read(x32, "ffn", layer.ffn_norm)
         f32 = layer.feed_forward.forward(d, None, ctx)
-        K.streams_write(x32, f32, self.w["ffn", "mix"], self.w["ffn", "out"])
+        self._last_write(x32, f32, "ffn", then, ctx)
         return x32
