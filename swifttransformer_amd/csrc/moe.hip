@@ -26,14 +26,27 @@ constexpr int kMaxTop = 16;
 
 __global__ __launch_bounds__(256) void moe_route_kernel(
     int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ logits,
-    const int* __restrict__ token_item, int num_tokens, int experts, int top, int mode, int groups, int keep) {
-    const int t = blockIdx.x * 256 + threadIdx.x;
+    const int* __restrict__ token_item, int num_tokens, int experts, int top, int mode, int groups, int keep,
+    int stage) {
+    // The rows of the workgroup's tokens go to LDS first, read side by side (a thread that walked its own row in
+    // memory would wait for every logit by itself, several times over); rows are experts + 1 floats apart.
+    extern __shared__ float s_z[];
+    const int t0 = blockIdx.x * blockDim.x, t = t0 + threadIdx.x;
+    if (stage) {
+        const int n = min((int)blockDim.x, num_tokens - t0);
+        const float* src = logits + (int64_t)t0 * experts;
+        for (int i = threadIdx.x; i < n * experts; i += blockDim.x) {
+            const int r = i / experts;
+            s_z[r * (experts + 1) + (i - r * experts)] = src[i];
+        }
+        __syncthreads();
+    }
     if (t >= num_tokens) return;
     if (token_item && token_item[t] < 0) {
         for (int j = 0; j < top; ++j) { ids[(int64_t)t * top + j] = -1; weights[(int64_t)t * top + j] = 0.f; }
         return;
     }
-    const float* z = logits + (int64_t)t * experts;
+    const float* z = stage ? s_z + threadIdx.x * (experts + 1) : logits + (int64_t)t * experts;
     // mode 2: only the experts of the `keep` groups (of `groups` equal groups of neighbours) whose largest
     // logit is largest can be chosen; bit g of `open` says that group g is one of them
     uint64_t open = ~0ull;
@@ -52,27 +65,51 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
             open |= 1ull << best;
         }
     }
-    int chosen[kMaxTop];
-    for (int j = 0; j < top; ++j) {
-        int best = -1;
-        float bv = 0.f;
-        for (int e = 0; e < experts; ++e) {
-            bool taken = mode == 2 && !((open >> (e / per)) & 1);
-            for (int u = 0; u < j; ++u) taken |= chosen[u] == e;
-            const float v = z[e];
-            if (!taken && (best < 0 || v > bv)) { best = e; bv = v; }
-        }
-        chosen[j] = best;
-        ids[(int64_t)t * top + j] = best;
-        weights[(int64_t)t * top + j] = mode == 0 ? 1.f / (1.f + expf(-bv)) : bv;
-    }
+    // mode 2: the weights are the chosen experts' shares of the softmax over all experts, as they are
+    float m_all = 0.f, inv_sum = 1.f;
     if (mode == 2) {
-        // the weights are the chosen experts' shares of the softmax over all experts, as they are
-        float m = z[0], sum = 0.f;
-        for (int e = 1; e < experts; ++e) m = fmaxf(m, z[e]);
-        for (int e = 0; e < experts; ++e) sum += expf(z[e] - m);
-        float* w = weights + (int64_t)t * top;
-        for (int j = 0; j < top; ++j) w[j] = expf(w[j] - m) / sum;
+        m_all = z[0];
+        for (int e = 1; e < experts; ++e) m_all = fmaxf(m_all, z[e]);
+        float sum = 0.f;
+        for (int e = 0; e < experts; ++e) sum += expf(z[e] - m_all);
+        inv_sum = 1.f / sum;
+    }
+    auto weight_of = [&](float v) { return mode == 0 ? 1.f / (1.f + expf(-v)) : mode == 2 ? expf(v - m_all) * inv_sum : v; };
+    if (experts <= 64) {
+        // which experts can still be chosen, a bit each: no list of the chosen ones to walk
+        uint64_t free_ = experts == 64 ? ~0ull : (1ull << experts) - 1;
+        if (mode == 2 && keep < groups) {
+            const uint64_t one_group = per == 64 ? ~0ull : (1ull << per) - 1;
+            free_ = 0;
+            for (int g = 0; g < groups; ++g)
+                if ((open >> g) & 1) free_ |= one_group << (g * per);
+        }
+        for (int j = 0; j < top; ++j) {
+            int best = -1;
+            float bv = 0.f;
+            for (int e = 0; e < experts; ++e) {
+                const float v = z[e];
+                if (((free_ >> e) & 1) && (best < 0 || v > bv)) { best = e; bv = v; }
+            }
+            free_ &= ~(1ull << best);
+            ids[(int64_t)t * top + j] = best;
+            weights[(int64_t)t * top + j] = weight_of(bv);
+        }
+    } else {
+        int chosen[kMaxTop];
+        for (int j = 0; j < top; ++j) {
+            int best = -1;
+            float bv = 0.f;
+            for (int e = 0; e < experts; ++e) {
+                bool taken = mode == 2 && !((open >> (e / per)) & 1);
+                for (int u = 0; u < j; ++u) taken |= chosen[u] == e;
+                const float v = z[e];
+                if (!taken && (best < 0 || v > bv)) { best = e; bv = v; }
+            }
+            chosen[j] = best;
+            ids[(int64_t)t * top + j] = best;
+            weights[(int64_t)t * top + j] = weight_of(bv);
+        }
     }
     if (mode == 1) {
         // softmax over the chosen logits alone; the first chosen is the largest
@@ -460,8 +497,12 @@ extern "C" int st_moe_route(int* ids, float* weights, const float* logits, const
              kMaxTop, experts, top);
     ST_CHECK(ids && weights && logits, "moe_route: null operand");
     if (num_tokens == 0) return 0;
-    moe_route_kernel<<<(num_tokens + 255) / 256, 256, 0, stream>>>(ids, weights, logits, token_item, num_tokens,
-                                                                  experts, top, mode, groups, keep);
+    // workgroups of as many tokens as have their rows side by side in 48 KB of LDS (256, 64, or none staged)
+    const size_t row = (size_t)(experts + 1) * sizeof(float);
+    const int threads = 256 * row <= 48 * 1024 ? 256 : 64;
+    const int stage = threads * row <= 48 * 1024;
+    moe_route_kernel<<<(num_tokens + threads - 1) / threads, threads, stage ? threads * row : 0, stream>>>(
+        ids, weights, logits, token_item, num_tokens, experts, top, mode, groups, keep, stage);
     ST_LAUNCH_CHECK("moe_route");
     return 0;
 }

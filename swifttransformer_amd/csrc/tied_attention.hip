@@ -31,20 +31,27 @@ __global__ __launch_bounds__(256) void qk_norm_write_kernel(
         for (int i = threadIdx.x; i < heads * head_pad; i += 256) Elem<T>::store(oq + i, 0.f);
         return;
     }
+    // (the page's number is asked for before the sums: its trip to memory runs beside theirs)
+    const int page = write ? block_table[(int64_t)item * max_pages + pos / page_size] : -1;
     float sq = 0.f, sk = 0.f;
     for (int i = threadIdx.x; i < nq; i += 256) sq = fmaf(q[i], q[i], sq);
     for (int i = threadIdx.x; i < nk; i += 256) sk = fmaf(k[i], k[i], sk);
-    sq = block_sum(sq, red);
-    sk = block_sum(sk, red);
+    {   // both sums over the workgroup with one exchange through LDS
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        sq = wave_sum(sq);
+        sk = wave_sum(sk);
+        if (lane == 0) { red[wave] = sq; red[4 + wave] = sk; }
+        __syncthreads();
+        sq = red[0] + red[1] + red[2] + red[3];
+        sk = red[4] + red[5] + red[6] + red[7];
+    }
     const float rq = 1.f / sqrtf(sq / (float)nq + eps), rk = 1.f / sqrtf(sk / (float)nk + eps);
     for (int i = threadIdx.x; i < heads * head_pad; i += 256) {
         const int h = i / head_pad, d = i - h * head_pad;
         const int j = h * head_dim + d;
         Elem<T>::store(oq + i, d < head_dim ? q[j] * rq * gq[j] : 0.f);
     }
-    if (!write) return;
-    const int page = block_table[(int64_t)item * max_pages + pos / page_size];
-    if (page < 0) return;
+    if (!write || page < 0) return;
     const int64_t base = (int64_t)page * page_stride + (int64_t)(pos % page_size) * head_pad;
     for (int i = threadIdx.x; i < kv_heads * head_pad; i += 256) {
         const int h = i / head_pad, d = i - h * head_pad;
