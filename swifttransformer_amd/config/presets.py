@@ -179,10 +179,10 @@ def pupalix_preset(name: str, **overrides):
         if kind == "latent_attention":
             mixer = {"heads": heads, "dim": hd, "rot_dim": 32, "vdim": hd, "kv_rank": 128, "scale": float(hd + 32) ** -0.5,
                      "rot": {"base": 10000.0, "dims": 32,
-                             "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+                             "scaling": {"factor": 8.0, "original": 1024, "fast": 16.0, "slow": 2.0}}}
         elif kind == "attention":
             mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": hd, "vdim": hd, "scale": float(hd) ** -0.5,
-                     "softcap": 30.0, "mask": {"size": chunk}}
+                     "softcap": 50.0, "mask": {"size": chunk}}
         else:
             lh = max(1, heads // 8)
             mixer = {"heads": lh, "dim": hd, "vdim": 2 * hd, "decay": [1.0 - 2.0 ** (-5 - (j % 4)) for j in range(lh)]}

@@ -73,7 +73,7 @@ CONFIGS = {
                      _with(_latent(3, 10, 6, 14, 30, 0.35, base=50.0), _moe(4, 1, 20, groups=(2, 2)))]},
     "C": {"architecture": "Pupalix", "vocab": 61, "width": 128, "max_positions": 512, "norm": {"eps": 1e-5},
           "embedding": {"scale": 2.0}, "logit_scale": 0.7, "logit_softcap": 20.0, "loop": {"start": 0, "stop": 3, "times": 1},
-          "layers": [_with(_attention(8, 1, 32, 0.25, softcap=30.0, chunk=64), _moe(8, 1, 40, groups=(4, 1))),
+          "layers": [_with(_attention(8, 1, 32, 0.25, softcap=25.0, chunk=64), _moe(8, 1, 40, groups=(4, 1))),
                      _with(_lightning(4, 64, 16, [0.5, 0.9, 0.99, 1.0]), _dense(96)),
                      _with(_latent(8, 16, 16, 32, 64, 0.2, base=1000.0,
                                    scaling={"factor": 8.0, "original": 32, "fast": 8.0, "slow": 0.5}), None)]},
