@@ -185,9 +185,9 @@ class PupalixHyperParam:
             width=_need(d, "width", "the top level", (int,), 1),
             layers=layers,
             streams=int(_need(d, "streams", "the top level", (int,), 1)) if d.get("streams") is not None else 0,
-            embedding_scale=float(emb.get("scale", 1.0)),
+            embedding_scale=float(emb["scale"]) if emb.get("scale") is not None else 1.0,
             bigram=copy.deepcopy(emb.get("bigram")) or None,
-            logit_scale=float(d.get("logit_scale", 1.0)),
+            logit_scale=float(d["logit_scale"]) if d.get("logit_scale") is not None else 1.0,
             logit_softcap=float(d.get("logit_softcap") or 0.0),
             loop=copy.deepcopy(d.get("loop")) or None,
             norm_eps=float(_need(d.get("norm"), "eps", "norm", _NUM)),
