@@ -448,6 +448,23 @@ def test_greedy_generation_through_the_engine(models):
             assert row.max() - row[tok] <= 0.05 * row.std() + 0.02 * abs(row.max())
 
 
+def test_a_request_that_loses_its_pages_starts_again_from_cleared_state(models):
+    """A pool that cannot hold the requests together: the scheduler takes pages back from a running request, which is
+    computed again later in a slot that held another request's recurrent state and last token."""
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.sampling import SamplingParams
+    folder, cfg, w = models["A"]
+    prompts = [tiny.prompt(n, cfg["vocab"], 70 + i) for i, n in enumerate((30, 26, 21, 5))]
+    sp = SamplingParams(max_new_tokens=20, ignore_eos=True)
+    tight = Engine(folder, dtype="fp32", page_size=4, num_pages=19, max_seqs=2, max_batched_tokens=64, prefill_chunk=9)
+    outs = tight.generate(prompts, sp)
+    assert tight.stats.preemptions >= 1, "the pool was meant to run out"
+    for p, o in zip(prompts, outs):
+        assert o == plain.generate(cfg, w, p, 20), f"prompt of {len(p)} tokens"
+    tight.runner.manager.check_invariants()
+    assert tight.runner.manager.num_free_slots == 2
+
+
 def test_trace_replay_command_line_and_a_named_size(models, tmp_path):
     import json
     import subprocess
