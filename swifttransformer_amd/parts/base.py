@@ -26,10 +26,13 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
                 ``biases_scores`` (bool) and ``score_slopes(num_heads) -> float32 [num_heads]``: an
                 attention mixer adds slope * (key position - query position) to a head's scaled
                 scores when ``biases_scores`` is true
-  embedding     ``forward(ctx, position) -> x32``
+  embedding     ``forward(ctx, position) -> x32``; one that keeps something a request offers ``cache_need()`` (a
+                "state" need) and gets ``forward(ctx, position, cache=view)``
   head          ``forward(y_t) -> logits float32 [R, vocab]``
   arrangement   ``forward(x32, layer, ctx, cache, write) -> x32`` (with ``conv_cache=`` for a layer
-                that has a ``mixer_conv`` part)
+                that has a ``mixer_conv`` part); it may declare tensors of its own; ``reads_ahead`` True: it is
+                called with ``then=`` the layer that runs next (or None) and may leave that layer's first input
+                in ``ctx.read_ahead``.  Where ``ModelSpec.streams`` is set, x32 is [T, streams * hidden]
   token_conv    ``cache_need() -> CacheNeed``; ``forward(y32, ctx, cache) -> y_t``: a short causal
                 filter over time on what a mixer reads, with its last inputs as per-request state
   side_input    ``forward(x32, ctx, x_t=None) -> x32`` (``x_t``: the stream in the storage type, if at hand): what a layer adds to the stream after its feed-forward
